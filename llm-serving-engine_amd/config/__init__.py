@@ -1,5 +1,6 @@
 from .model import ArchitectureConfig, ConfigError, KeyReader, Qwen2Config
 from .dafutar import DafutarConfig
+from .katenex import KatenexConfig
 from .serving import CacheConfig, SchedulerConfig
 
 __all__ = [
@@ -7,6 +8,7 @@ __all__ = [
     "CacheConfig",
     "ConfigError",
     "DafutarConfig",
+    "KatenexConfig",
     "KeyReader",
     "Qwen2Config",
     "SchedulerConfig",

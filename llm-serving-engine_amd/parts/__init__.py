@@ -17,7 +17,7 @@ from .base import (
     TensorSpec,
 )
 from .norm import LayerNorm, LayerNormSpec, RMSNorm, RMSNormSpec
-from .position import HeadLayout, NoPositionSpec, PositionEncoding, Rotary, RotarySpec, WavelengthScaling, YarnScaling, rotary_frequencies
+from .position import HeadLayout, LinearScaling, NoPositionSpec, PositionEncoding, Rotary, RotarySpec, WavelengthScaling, YarnScaling, rotary_frequencies
 from .attention import Attention, AttentionSpec, Mixer
 from .feed_forward import FeedForward, GatedMLP, GatedMLPSpec
 from .block import Block, OutputNormBlock, OutputNormBlockSpec, PreNormBlock, PreNormBlockSpec
@@ -27,5 +27,8 @@ from .delta import GatedDelta, GatedDeltaSpec
 from .experts import RoutedExperts, RoutedExpertsSpec
 from .normed_attention import NormedAttention, NormedAttentionSpec
 from .decay_attention import DecayAttention, DecayAttentionSpec
+from .hyper import HyperBlock, HyperBlockSpec, PendingWrite, StreamCopies, StreamCopiesSpec, StreamNorm, StreamNormSpec
+from .recurrent import GatedRecurrence, GatedRecurrenceSpec
+from .parallel import ParallelMixers, ParallelMixersSpec
 
 __all__ = [name for name in dir() if not name.startswith("_")]

@@ -124,8 +124,9 @@ class DecoderModel:
 
     def _run_layers(self, batch, cells: list):
         hidden = self.kernels.embedding(self.embedding, batch.token_ids)
-        for part in self.input_parts:
-            part.forward(hidden, batch)
+        for part in self.input_parts:  # (in place, or a new stream of another shape: copies side by side)
+            changed = part.forward(hidden, batch)
+            hidden = hidden if changed is None else changed
         embedded = hidden.clone() if self.pass_entry is not None else None  # the layers add into `hidden` in place
         delta = None
         for index, (run, cell) in enumerate(zip(self.spec.run_order, cells)):
@@ -146,6 +147,8 @@ class DecoderModel:
         hidden, delta = self._run_layers(batch, cells)
         if getattr(batch, "every_row_wanted", False):  # the final norm adds the last layer's delta itself
             normed = self.final_norm.forward(hidden, delta)
+        elif hasattr(self.final_norm, "forward_rows"):  # a norm that reads the wanted rows of the stream itself
+            normed = self.final_norm.forward_rows(hidden, delta, batch.logit_rows)
         else:
             rows = self.kernels.gather_rows(hidden, delta, batch.logit_rows)
             normed = self.final_norm.forward(rows, None)

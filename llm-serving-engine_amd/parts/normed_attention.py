@@ -10,7 +10,7 @@ import torch
 
 from .attention import Mixer
 from .base import MIXERS, PagedKeyValue, TensorSpec
-from .position import HeadLayout, WavelengthScaling, YarnScaling, rotary_frequencies
+from .position import HeadLayout, LinearScaling, WavelengthScaling, YarnScaling, rotary_frequencies
 
 
 @dataclass(frozen=True)
@@ -21,7 +21,8 @@ class NormedAttentionSpec:
     `norm`: "head" (RMS norm of every query and key head with one weight of `dim` for all heads), "row" (RMS norm of
     the whole query projection and of the whole key projection, with weights as long as they), or None.
     `rot_dims`: the first so many dimensions of every query and key head turn by the position, in adjacent pairs
-    (2i, 2i + 1), with the frequencies theta^(-2i / rot_dims) stretched by `scaling`; 0: positions do not enter.
+    (2i, 2i + 1) or, with `pairing` "half", in pairs (i, i + rot_dims / 2), with the frequencies theta^(-2i / rot_dims)
+    stretched by `scaling`; 0: positions do not enter.
     `soft_cap`: scores become cap * tanh(score / cap).  `sink`: a learned number a head whose exponential is added
     once to the softmax's denominator.  `gate`: head h's result times sigmoid of row h of a product of the mixer's input.
     `values`: None, "give" (the step's values are shown to later layers under `values_name`) or "take" (v <- (1 - a) v
@@ -39,7 +40,8 @@ class NormedAttentionSpec:
     norm: str | None = "head"
     rot_dims: int = 0
     theta: float = 10000.0
-    scaling: YarnScaling | WavelengthScaling | None = None
+    scaling: YarnScaling | WavelengthScaling | LinearScaling | None = None
+    pairing: str = "adjacent"
     soft_cap: float | None = None
     sink: bool = False
     gate: bool = False
@@ -96,6 +98,8 @@ class NormedAttention(Mixer):
             raise ValueError("normed attention: the query heads are a multiple of the key/value heads")
         if spec.norm not in (None, "head", "row") or spec.values not in (None, "give", "take"):
             raise ValueError("normed attention: norm is 'head', 'row' or None; values 'give', 'take' or None")
+        if spec.pairing not in ("adjacent", "half"):
+            raise ValueError("normed attention: pairing is 'adjacent' or 'half'")
         if spec.rot_dims % 2 or spec.rot_dims > spec.dim:
             raise ValueError("normed attention: the rotated dimensions are an even number within dim")
         heads, width = spec.num_heads, spec.head_width
@@ -145,6 +149,7 @@ class NormedAttention(Mixer):
             spec.norm, self.q_norm, self.k_norm, spec.eps, table, spec.rot_dims,
             given[0] if given else None, given[1] if given else 0, self.blend,
             batch=batch, cell=None if plain else cell,  # (with plain scores the attention below stores, and may fuse that)
+            pairing=spec.pairing,
         )
         if plain:
             return kernels.rotate_store_attend(rows, self.layout, batch, cell, None, "none", spec.scale, spec.window, project=self.out)

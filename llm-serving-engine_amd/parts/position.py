@@ -119,13 +119,22 @@ class WavelengthScaling:
     original: float
 
 
-def rotary_frequencies(dims: int, theta: float, scaling: "YarnScaling | WavelengthScaling | None" = None) -> tuple[torch.Tensor, float]:
+@dataclass(frozen=True)
+class LinearScaling:
+    """Every frequency divided by `factor` (positions counted in steps of 1 / factor).  Cosines and sines stay as they are."""
+
+    factor: float
+
+
+def rotary_frequencies(dims: int, theta: float, scaling: "YarnScaling | WavelengthScaling | LinearScaling | None" = None) -> tuple[torch.Tensor, float]:
     """(float32 frequencies [dims / 2] of pair i, theta^(-2i / dims), stretched by `scaling`; what the cosines
     and sines are multiplied by).  Computed in float64 and rounded once."""
     index = torch.arange(dims // 2, dtype=torch.float64)
     plain = float(theta) ** (-2.0 * index / dims)
     if scaling is None:
         return plain.to(torch.float32), 1.0
+    if isinstance(scaling, LinearScaling):
+        return (plain / float(scaling.factor)).to(torch.float32), 1.0
     if isinstance(scaling, WavelengthScaling):
         wavelength = 2.0 * math.pi / plain
         share = ((scaling.original / wavelength - scaling.low) / (scaling.high - scaling.low)).clamp(0.0, 1.0)

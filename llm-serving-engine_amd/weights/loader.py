@@ -126,11 +126,18 @@ def load_model_folder(
     folder = Path(folder)
     dtype = run_dtype(dtype)
     architecture, config = read_config(folder)
-    spec = architecture.build_spec(config)
-    expected = spec.tensors()
     files = sorted(folder.glob("*.safetensors"))
     if not files:
         raise FileNotFoundError(f"no safetensors files under {folder}")  # `checkpoint.py:47-48`
+    found: dict[str, torch.Tensor] = {}
+    for path in files:
+        with safe_open(str(path), framework="pt", device="cpu") as source:
+            for source_name in source.keys():
+                found[source_name] = source.get_tensor(source_name)
+    if hasattr(config, "with_sizes_of"):  # sizes that config.json leaves to the tensors' shapes
+        config = config.with_sizes_of({name: tuple(tensor.shape) for name, tensor in found.items()})
+    spec = architecture.build_spec(config)
+    expected = spec.tensors()
 
     def model_name(name: str) -> str:
         if name in expected:
@@ -140,11 +147,6 @@ def load_model_folder(
                 return candidate
         return name
 
-    found: dict[str, torch.Tensor] = {}
-    for path in files:
-        with safe_open(str(path), framework="pt", device="cpu") as source:
-            for source_name in source.keys():
-                found[source_name] = source.get_tensor(source_name)
     if architecture.adapt_tensors is not None:  # the files name or cut their tensors otherwise than the parts do
         found = architecture.adapt_tensors(found, config)
     found = {model_name(name): tensor for name, tensor in found.items()}

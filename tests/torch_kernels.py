@@ -220,8 +220,8 @@ class TorchKernels:
 
     # ------------------------------------------------------------------ the gated delta rule
 
-    def causal_conv(self, x, channels, taps, activation, batch, window):
-        assert activation == "silu"
+    def causal_conv(self, x, channels, taps, activation, batch, window, bias=None):
+        assert activation in ("silu", "none")
         width = taps.shape[1]
         out = torch.zeros((x.shape[0], channels))
         row = 0
@@ -234,9 +234,11 @@ class TorchKernels:
             if window is not None:
                 window[chunk.slot] = line[-(width - 1):]
             row += chunk.count
-        return torch.nn.functional.silu(out).to(self.dtype)
+        if bias is not None:
+            out = out + bias.float()
+        return (torch.nn.functional.silu(out) if activation == "silu" else out).to(self.dtype)
 
-    def gated_delta_rule(self, mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state):
+    def gated_delta_rule(self, mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state, channel_steps=None):
         tokens = mixed.shape[0]
         q = mixed[:, : kv_heads * dim].float().view(tokens, kv_heads, dim)
         k = mixed[:, kv_heads * dim : 2 * kv_heads * dim].float().view(tokens, kv_heads, dim)
@@ -244,7 +246,12 @@ class TorchKernels:
         q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * dim**-0.5
         k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
         beta = torch.sigmoid(controls[:, :heads].float())
-        decay = torch.exp(-torch.exp(rate.float()) * torch.nn.functional.softplus(controls[:, heads:].float() + step_bias.float()))
+        if channel_steps is None:
+            decay = torch.exp(-torch.exp(rate.float()) * torch.nn.functional.softplus(controls[:, heads:].float() + step_bias.float()))
+            decay = decay.view(tokens, heads, 1, 1)
+        else:  # a decay for every key channel of every head
+            steps = torch.nn.functional.softplus(channel_steps[:, : heads * dim].float() + step_bias.float()).view(tokens, heads, dim)
+            decay = torch.exp(-torch.exp(rate.float()).view(1, heads, 1) * steps).view(tokens, heads, dim, 1)
         out = torch.zeros((tokens, heads, vdim))
         row = 0
         for chunk in batch.chunks:
@@ -252,7 +259,7 @@ class TorchKernels:
             for t in range(row, row + chunk.count):
                 kt = k[t].repeat_interleave(heads // kv_heads, dim=0)
                 qt = q[t].repeat_interleave(heads // kv_heads, dim=0)
-                S *= decay[t].view(heads, 1, 1)
+                S *= decay[t]
                 u = beta[t].view(heads, 1) * (v[t] - torch.einsum("hdv,hd->hv", S, kt))
                 S += torch.einsum("hd,hv->hdv", kt, u)
                 out[t] = torch.einsum("hdv,hd->hv", S, qt)
@@ -280,7 +287,7 @@ class TorchKernels:
         return hidden if self.dtype == torch.float32 else hidden.to(self.dtype)
 
     def assemble_heads(self, x, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, q_weight, k_weight, eps,
-                       table, rot_dims, other=None, other_first=0, blend=0.0, batch=None, cell=None):
+                       table, rot_dims, other=None, other_first=0, blend=0.0, batch=None, cell=None, pairing="adjacent"):
         tokens = x.shape[0]
         out = torch.zeros((tokens, heads + 2 * kv_heads, width))
 
@@ -293,10 +300,11 @@ class TorchKernels:
                 part = part * torch.rsqrt(part.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
             if rot_dims:
                 cos, sin = table[:, None, :, 0], table[:, None, :, 1]
-                a, b = part[..., 0:rot_dims:2], part[..., 1:rot_dims:2]
+                first, second = (slice(0, rot_dims, 2), slice(1, rot_dims, 2)) if pairing == "adjacent" else (slice(0, rot_dims // 2), slice(rot_dims // 2, rot_dims))
+                a, b = part[..., first], part[..., second]
                 turned = part.clone()
-                turned[..., 0:rot_dims:2] = a * cos - b * sin
-                turned[..., 1:rot_dims:2] = b * cos + a * sin
+                turned[..., first] = a * cos - b * sin
+                turned[..., second] = b * cos + a * sin
                 part = turned
             return part
 
@@ -342,28 +350,85 @@ class TorchKernels:
 
     # ------------------------------------------------------------------ routed experts
 
-    def route(self, scores, experts, correction, top, scale, scoring):
-        assert scoring == "sigmoid"
-        squashed = torch.sigmoid(scores[:, :experts].float())
-        choice = squashed + correction.float()
+    def route(self, scores, experts, correction, top, scale, scoring, groups=1, keep_groups=1, renormalise=False):
+        z = scores[:, :experts].float()
+        squashed = torch.sigmoid(z) if scoring == "sigmoid" else torch.softmax(z, dim=-1)
+        assert scoring in ("sigmoid", "softmax")
+        choice = squashed + correction.float() if correction is not None else squashed.clone()
+        if groups > 1:  # only experts of the best groups can be chosen; a group's score is its largest
+            best = choice.view(-1, groups, experts // groups).max(-1).values
+            kept = torch.sort(best, dim=-1, descending=True, stable=True).indices[:, :keep_groups]
+            allowed = torch.zeros_like(best, dtype=torch.bool).scatter_(1, kept, True).repeat_interleave(experts // groups, dim=1)
+            choice = torch.where(allowed, choice, torch.full_like(choice, -math.inf))
         chosen = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
-        return chosen.to(torch.int32), (squashed.gather(1, chosen) * scale).float()
+        weights = squashed.gather(1, chosen)
+        if renormalise:
+            weights = weights / (weights.sum(-1, keepdim=True) + 1e-20)
+        return chosen.to(torch.int32), (weights * scale).float()
 
-    def prepare_experts(self, ups, downs, activation):
-        return (torch.stack([w.float() for w in ups]), torch.stack([w.float() for w in downs]), activation)
+    def prepare_experts(self, ups, downs, activation, gates=None):
+        stacked = torch.stack([w.float() for w in gates]) if gates is not None else None
+        return (torch.stack([w.float() for w in ups]), torch.stack([w.float() for w in downs]), activation, stacked)
 
-    def conv_gated_delta_rule(self, projected, channels, taps, activation, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, window, state):
+    def conv_gated_delta_rule(self, projected, channels, taps, activation, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, window, state,
+                              channel_steps=None):
         mixed = self.causal_conv(projected, channels, taps, activation, batch, window)
-        return self.gated_delta_rule(mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state)
+        return self.gated_delta_rule(mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state, channel_steps=channel_steps)
 
     def expert_feed_forward(self, x, experts, chosen, weights, shared=None, gates=None, gate_column=0):
-        ups, downs, activation = experts
+        ups, downs, activation, gate_weights = experts
         out = torch.zeros((x.shape[0], downs.shape[1]))
         for t in range(x.shape[0]):
             for slot in range(chosen.shape[1]):
                 e = int(chosen[t, slot])
-                inner = self.activate((x[t].float() @ ups[e].T).to(self.dtype), activation).float()
+                if gate_weights is None:
+                    inner = self.activate((x[t].float() @ ups[e].T).to(self.dtype), activation).float()
+                else:  # act(gate x) * (up x), both rounded to the run dtype before
+                    gate = self.activate((x[t].float() @ gate_weights[e].T).to(self.dtype), activation).float()
+                    inner = (gate * (x[t].float() @ ups[e].T).to(self.dtype).float()).to(self.dtype).float()
                 out[t] += weights[t, slot] * (inner @ downs[e].T)
         if shared is not None:
-            out += torch.sigmoid(gates[:, gate_column : gate_column + 1].float()) * shared
+            out += torch.sigmoid(gates[:, gate_column : gate_column + 1].float()) * shared if gates is not None else shared
         return out
+
+    # ------------------------------------------------------------------ copies of the stream, a diagonal recurrence, weighted sums
+
+    def stream_copies(self, hidden, copies, scale):
+        return (hidden * scale).repeat(1, copies)
+
+    def stream_norm(self, streams, pending, read, weight, eps, rows=None):
+        copies = read.shape[0]
+        now = streams if pending is None else pending.applied(streams)
+        if rows is None:
+            if pending is not None:
+                streams.copy_(now)
+        else:
+            now = now[rows.long()]
+        u = torch.einsum("s,nsh->nh", read.float(), now.view(now.shape[0], copies, -1))
+        return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(self.dtype)
+
+    def gated_recurrence(self, u, gates, gate_bias, rates, branch, branch_first, activation, blocks, batch, state):
+        assert activation == "gelu_tanh"
+        tokens, width = u.shape
+        part = width // blocks
+        z = gates.float().view(tokens, blocks, 2 * part) + gate_bias.float()
+        r = torch.sigmoid(z[..., :part]).reshape(tokens, width)
+        i = torch.sigmoid(z[..., part:]).reshape(tokens, width)
+        a = torch.exp(rates.float() * r)
+        push = torch.sqrt(1.0 - a * a) * i * u.float()
+        y = torch.nn.functional.gelu(branch[:, branch_first : branch_first + width].float(), approximate="tanh")
+        out = torch.zeros((tokens, width))
+        row = 0
+        for chunk in batch.chunks:
+            S = state[chunk.slot]
+            for t in range(row, row + chunk.count):
+                S.copy_(a[t] * S + push[t])
+                out[t] = S * y[t]
+            row += chunk.count
+        return out.to(self.dtype)
+
+    def add_scaled(self, a, a_scale, b, b_scale):
+        total = a_scale * (a if a.ndim == 2 else a.sum(0))
+        if b is not None:
+            total = total + b_scale * (b if b.ndim == 2 else b.sum(0))
+        return total
