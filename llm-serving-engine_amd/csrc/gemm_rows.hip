@@ -356,22 +356,71 @@ extern "C" int llmserve_headwise_linear(const void* x, int is_float, int rows, i
 }
 
 // ---------------------------------------------------------------------------- routing
-// One wave a token: s_e = sigmoid(z[t, e]); the `top` experts with the largest s_e + correction_e, the lower index
-// first among equals; chosen[t, i] and weight[t, i] = scale * s_e (no renormalising).  Lane l keeps the experts
-// l, l + 64, ...; a pick is the wave's best of the lanes' best, which is then struck out.
+// One wave a token: s_e = sigmoid(z[t, e]) or softmax(z[t, :])_e; the `top` experts with the largest s_e + correction_e,
+// the lower index first among equals, taken from the experts of the `keep` best of `groups` equal groups of neighbours;
+// chosen[t, i] and weight[t, i] = scale * s_e, with `renormalise` scale * s_e / (sum of the chosen s + 1e-20).  Lane l
+// keeps the experts l, l + 64, ...; a pick is the wave's best of the lanes' best, which is then struck out.
 #define ROUTE_PER_LANE 16
 __global__ __launch_bounds__(WAVE) void route_kernel(const float* __restrict__ z, int z_stride, int experts,
                                                      const float* __restrict__ correction, int top, float scale,
-                                                     int* __restrict__ chosen, float* __restrict__ weight) {
+                                                     int* __restrict__ chosen, float* __restrict__ weight, int softmax,
+                                                     int groups, int keep, int renormalise) {
+  __shared__ float by_expert[ROUTE_PER_LANE * WAVE];
+  __shared__ float by_group[ROUTE_PER_LANE * WAVE];
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* row = z + (size_t)t * z_stride;
   float score[ROUTE_PER_LANE], choice[ROUTE_PER_LANE];
+  float top_z = -INFINITY, total = 1.f;
+  if (softmax) {  // over all experts: exp(z - max) / sum
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+      const int e = lane + j * WAVE;
+      if (e < experts) top_z = fmaxf(top_z, row[e]);
+    }
+    top_z = wave_max(top_z);
+    total = 0.f;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+      const int e = lane + j * WAVE;
+      score[j] = e < experts ? expf(row[e] - top_z) : 0.f;
+      total += score[j];
+    }
+    total = wave_sum(total);
+  }
 #pragma unroll
   for (int j = 0; j < ROUTE_PER_LANE; ++j) {
     const int e = lane + j * WAVE;
-    score[j] = e < experts ? 1.f / (1.f + expf(-row[e])) : 0.f;
-    choice[j] = e < experts ? score[j] + correction[e] : -INFINITY;
+    if (softmax) score[j] = score[j] / total;
+    else score[j] = e < experts ? 1.f / (1.f + expf(-row[e])) : 0.f;
+    choice[j] = e < experts ? score[j] + (correction ? correction[e] : 0.f) : -INFINITY;
   }
+  if (groups > 1) {
+    // Only the experts of the `keep` best groups of neighbours stay; a group's score is its largest (the lower index
+    // among equals, as everywhere here).
+    const int size = experts / groups;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; ++j)
+      if (lane + j * WAVE < experts) by_expert[lane + j * WAVE] = choice[j];
+    __syncthreads();
+    for (int g = lane; g < groups; g += WAVE) {
+      float best = -INFINITY;
+      for (int i = 0; i < size; ++i) best = fmaxf(best, by_expert[g * size + i]);
+      by_group[g] = best;
+    }
+    __syncthreads();
+    // group g stays if fewer than `keep` groups come before it in the order (score descending, index ascending)
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+      const int e = lane + j * WAVE;
+      if (e >= experts) continue;
+      const int g = e / size;
+      const float mine = by_group[g];
+      int before = 0;
+      for (int o = 0; o < groups; ++o) before += (by_group[o] > mine || (by_group[o] == mine && o < g)) ? 1 : 0;
+      if (before >= keep) choice[j] = -INFINITY;
+    }
+  }
+  float sum = 0.f;
   for (int i = 0; i < top; ++i) {
     float best = -INFINITY, best_score = 0.f;
     int best_expert = 0x7fffffff;
@@ -388,21 +437,28 @@ __global__ __launch_bounds__(WAVE) void route_kernel(const float* __restrict__ z
         best = other; best_score = other_score; best_expert = other_expert;
       }
     }
+    sum += best_score;
     if (lane == 0) {
       chosen[(size_t)t * top + i] = best_expert;
-      weight[(size_t)t * top + i] = scale * best_score;
+      weight[(size_t)t * top + i] = renormalise ? best_score : scale * best_score;
     }
 #pragma unroll
     for (int j = 0; j < ROUTE_PER_LANE; ++j)
       if (lane + j * WAVE == best_expert) choice[j] = -INFINITY;
   }
+  if (renormalise && lane == 0)  // (the lane reads back what it wrote itself)
+    for (int i = 0; i < top; ++i) weight[(size_t)t * top + i] = weight[(size_t)t * top + i] / (sum + 1e-20f) * scale;
 }
 
+// `correction` may be null (the choice is by score alone).  softmax 0: sigmoid of each score; 1: softmax over all experts.
 extern "C" int llmserve_route(const float* z, int z_stride, int experts, const float* correction, int top, float scale,
-                              int* chosen, float* weight, int tokens, hipStream_t stream) {
+                              int* chosen, float* weight, int tokens, int softmax, int groups, int keep, int renormalise,
+                              hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (experts < 1 || top < 1 || top > experts || experts > z_stride || experts > ROUTE_PER_LANE * WAVE) return ERR_BAD_ARGUMENT;
-  hipLaunchKernelGGL(route_kernel, dim3(tokens), dim3(WAVE), 0, stream, z, z_stride, experts, correction, top, scale, chosen, weight);
+  if (groups < 1 || experts % groups || keep < 1 || keep > groups || top > keep * (experts / groups)) return ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(route_kernel, dim3(tokens), dim3(WAVE), 0, stream, z, z_stride, experts, correction, top, scale, chosen, weight,
+                     softmax, groups, keep, renormalise);
   return LAUNCH_STATUS();
 }
 
@@ -570,7 +626,7 @@ __global__ void combine_pairs_kernel(const float* __restrict__ rows, const int* 
                                      int top, float* __restrict__ out, int width, const float* __restrict__ shared,
                                      const float* __restrict__ gates, int gate_stride, int gate_column) {
   const int t = blockIdx.x;
-  const float gate = shared ? 1.f / (1.f + expf(-gates[(size_t)t * gate_stride + gate_column])) : 0.f;
+  const float gate = shared ? (gates ? 1.f / (1.f + expf(-gates[(size_t)t * gate_stride + gate_column])) : 1.f) : 0.f;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float sum = 0.f;
     for (int i = 0; i < top; ++i) sum += weight[(size_t)t * top + i] * rows[(size_t)place[(size_t)t * top + i] * width + c];
@@ -583,7 +639,7 @@ extern "C" int llmserve_combine_pairs(const float* rows, const int* place, const
                                       int width, const float* shared, const float* gates, int gate_stride, int gate_column,
                                       hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (shared && (!gates || gate_column < 0 || gate_column >= gate_stride)) return ERR_BAD_ARGUMENT;
+  if (shared && gates && (gate_column < 0 || gate_column >= gate_stride)) return ERR_BAD_ARGUMENT;  // (no gates: the shared rows are added as they are)
   hipLaunchKernelGGL(combine_pairs_kernel, dim3(tokens), dim3(256), 0, stream, rows, place, weight, top, out, width, shared, gates,
                      gate_stride, gate_column);
   return LAUNCH_STATUS();

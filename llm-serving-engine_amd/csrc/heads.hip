@@ -176,12 +176,13 @@ extern "C" int llmserve_add_normed(float* hidden, const float* update, int parts
 // ---------------------------------------------------------------------------- heads put together for the attention
 // One block per token, a wave a head at a time.  A query or key head of `dim` is RMS-normed (norm 1: by itself, the
 // weight of `dim` shared by the heads; 2: all heads of the projection together, the weight as long as they; 0: not),
-// its first `rot_dims` dimensions are turned in pairs (2i, 2i + 1) by (cos, sin) of table[token][i], and it is written
+// its first `rot_dims` dimensions are turned in pairs (2i, 2i + 1), or with `pairing` 2 in pairs (i, i + rot_dims / 2), by
+// (cos, sin) of table[token][i], and it is written
 // `width` wide, zeros beyond `dim`.  A value head of `vdim` is blended with the same columns of `other` and written
 // `width` wide.  The output row is [heads | kv_heads | kv_heads] heads of `width`; the keys and values may go to
 // their pages in the same kernel (a step of single tokens: one launch less).
 struct HeadSizes {
-  int x_width, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, rot_dims, other_width, other_first;
+  int x_width, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, rot_dims, other_width, other_first, pairing;
 };
 
 template <typename T>
@@ -233,10 +234,14 @@ __global__ __launch_bounds__(1024) void assemble_heads_kernel(const T* __restric
         if (z.norm) mine *= load_as_float(weight, weight_is_float, weight_first + e);
         result = mine;
         if (e < z.rot_dims) {
-          float partner = to_float(src[e ^ 1]) * scale;
-          if (z.norm) partner *= load_as_float(weight, weight_is_float, weight_first + (e ^ 1));
-          const float c = angles[e & ~1], s = angles[(e & ~1) + 1];
-          result = (e & 1) ? mine * c + partner * s : mine * c - partner * s;
+          const int half = z.rot_dims / 2;
+          const int other_e = z.pairing == 2 ? (e < half ? e + half : e - half) : (e ^ 1);
+          const int pair = z.pairing == 2 ? (e < half ? e : e - half) : (e >> 1);
+          const bool second = z.pairing == 2 ? e >= half : (e & 1);
+          float partner = to_float(src[other_e]) * scale;
+          if (z.norm) partner *= load_as_float(weight, weight_is_float, weight_first + other_e);
+          const float c = angles[2 * pair], s = angles[2 * pair + 1];
+          result = second ? mine * c + partner * s : mine * c - partner * s;
         }
       }
       dst[(size_t)unit * z.width + e] = from_float<T>(result);
@@ -275,14 +280,15 @@ extern "C" int llmserve_assemble_heads(const void* x, int is_float, int tokens, 
                                        int heads, int kv_heads, int dim, int vdim, int width, int norm, const void* q_weight,
                                        const void* k_weight, int weight_is_float, float eps, const float* table, int rot_dims,
                                        const void* other, int other_width, int other_first, float blend, void* out,
-                                       void* keys, void* values, const int* slots, int page_size, hipStream_t stream) {
+                                       void* keys, void* values, const int* slots, int page_size, int pairing, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  if (pairing < 1 || pairing > 2) return ERR_BAD_ARGUMENT;
   if (heads < 1 || kv_heads < 1 || dim < 1 || vdim < 1 || width < dim || width < vdim || norm < 0 || norm > 2 ||
       (norm && (!q_weight || !k_weight)) || rot_dims < 0 || rot_dims % 2 || rot_dims > dim || (rot_dims && !table) ||
       q_first < 0 || k_first < 0 || v_first < 0 || q_first + heads * dim > x_width || k_first + kv_heads * dim > x_width ||
       v_first + kv_heads * vdim > x_width || (other && (other_first < 0 || other_first + kv_heads * vdim > other_width)))
     return ERR_BAD_ARGUMENT;
-  const HeadSizes z = {x_width, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, rot_dims, other_width, other_first};
+  const HeadSizes z = {x_width, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, rot_dims, other_width, other_first, pairing};
   if (slots && (!keys || !values || page_size < 1)) return ERR_BAD_ARGUMENT;
   // a wave a head where there are up to sixteen of them (a step of few tokens is as long as its longest workgroup)
   const int threads = WAVE * max(4, min(16, heads + kv_heads));

@@ -80,21 +80,25 @@ _SIGNATURES = {
     "llmserve_activate": "ppiiiip",
     "llmserve_add_gated_rows": "pppiiiip",
     "llmserve_headwise_linear": "piiiiipiiipiiip",
-    "llmserve_route": "piipifppip",
+    "llmserve_route": "piipifppiiiiip",
     "llmserve_sort_pairs": "piipppiip",
     "llmserve_expert_product": "pipipiipiipiip",
     "llmserve_combine_pairs": "pppipiippiip",
-    "llmserve_conv_gated_delta_rule": "piiipipppppiiiippiiipppppp",
-    "llmserve_causal_conv": "piiiipipppippp",
-    "llmserve_gated_delta_rule": "pipppiiiippiiippppp",
+    "llmserve_conv_gated_delta_rule": "piiipipppppiiiippiiippppppip",
+    "llmserve_causal_conv": "piiiipipppipppip",
+    "llmserve_gated_delta_rule": "pipppiiiippiiipppppip",
     "llmserve_delta_line": "i",
-    "llmserve_gated_head_norm": "ppiiipifiiiipp",
+    "llmserve_gated_head_norm": "ppiiipifiiiiipp",
     "llmserve_stream_rows": "ppipiip",
     "llmserve_add_normed": "ppipipiiifp",
-    "llmserve_assemble_heads": "piiiiiiiiiiiippifpipiifppppip",
+    "llmserve_assemble_heads": "piiiiiiiiiiiippifpipiifppppiip",
     "llmserve_scale_heads": "piiiipiip",
     "llmserve_soft_cap": "piifp",
     "llmserve_decay_attention": "piiiiiiiiipppiippiipp",
+    "llmserve_stream_copies": "ppiiifp",
+    "llmserve_stream_norm": "ppiippppipipiiifp",
+    "llmserve_add_scaled": "pifpifpiip",
+    "llmserve_gated_recurrence": "pippppiiiippiippp",
 }
 _TYPES = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
 
@@ -1177,35 +1181,41 @@ class HipKernels:
         _check(status, "headwise_linear")
         return out
 
-    def route(self, scores, experts: int, correction, top: int, scale: float, scoring: str):
-        if scoring != "sigmoid":
+    def route(self, scores, experts: int, correction, top: int, scale: float, scoring: str, groups: int = 1, keep_groups: int = 1,
+              renormalise: bool = False):
+        if scoring not in ("sigmoid", "softmax"):
             raise KernelError(f"route: no kernel scores experts by {scoring!r}")
-        if scores.dtype != torch.float32 or correction.dtype != torch.float32 or correction.shape != (experts,):
+        if scores.dtype != torch.float32 or (correction is not None and (correction.dtype != torch.float32 or correction.shape != (experts,))):
             raise KernelError("route: float32 scores and one float32 correction an expert")
         tokens = scores.shape[0]
         chosen = self._empty((tokens, top), torch.int32)
         weights = self._empty((tokens, top), torch.float32)
         status = self._library_of("gemm_rows").llmserve_route(
             _pointer(scores), scores.shape[1], experts, _pointer(correction), top, float(scale), _pointer(chosen), _pointer(weights),
-            tokens, self._stream,
+            tokens, 1 if scoring == "softmax" else 0, groups, keep_groups, 1 if renormalise else 0, self._stream,
         )
         _check(status, "route")
         return chosen, weights
 
-    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str):
-        """The experts' weights stacked: ([experts, size, hidden], [experts, hidden, size], activation)."""
+    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str, gates: list[torch.Tensor] | None = None):
+        """The experts' weights stacked: ([experts, size, hidden], [experts, hidden, size], activation, gated).  With `gates`
+        an expert's gate and up rows alternate (gate_0, up_0, gate_1, ...: [experts, 2 size, hidden]), so that a row of the
+        first product holds every gate beside its up."""
         if activation not in _ACTIVATIONS:
             raise KernelError(f"experts: no kernel applies the activation {activation!r} (known: {', '.join(_ACTIVATIONS)})")
-        return torch.stack(list(ups)).contiguous(), torch.stack(list(downs)).contiguous(), activation
+        if gates is None:
+            return torch.stack(list(ups)).contiguous(), torch.stack(list(downs)).contiguous(), activation, False
+        both = torch.stack([torch.stack([gate, up], dim=1).reshape(2 * up.shape[0], up.shape[1]) for gate, up in zip(gates, ups)])
+        return both.contiguous(), torch.stack(list(downs)).contiguous(), activation, True
 
     def expert_feed_forward(self, x, experts, chosen, weights, shared=None, gates=None, gate_column: int = 0) -> torch.Tensor:
         """sum over a token's chosen experts of weight * down(act(up x)), float32 [T, hidden].  The (token, choice)
         pairs are sorted by expert on the device, the two products run over tiles of one expert's rows, and a last
         kernel adds each token's rows up in the order of its choices; with `shared` (float32 [T, hidden]) it adds
         sigmoid(gates[:, gate_column]) * shared as well."""
-        ups, downs, activation = experts
+        ups, downs, activation, gated = experts
         tokens, top = chosen.shape
-        count, size, hidden = ups.shape
+        count, size, hidden = ups.shape  # (gated: `size` counts gate and up rows, twice the experts' width)
         if x.dtype != ups.dtype or x.shape != (tokens, hidden):
             raise KernelError("experts: rows and weights are of one type")
         library = self._library_of("gemm_rows")
@@ -1223,24 +1233,32 @@ class HipKernels:
         inner = self._empty((pairs, size), x.dtype)
         _check(library.llmserve_expert_product(
             _pointer(x), _is_float(x), _pointer(order), top, _pointer(ups), size, hidden, _pointer(tiles), capacity, tile_rows, _pointer(inner),
-            _is_float(inner), _ACTIVATIONS[activation], self._stream), "experts: first product")
+            _is_float(inner), -1 if gated else _ACTIVATIONS[activation], self._stream), "experts: first product")
+        if gated:  # act(gate) * up of the neighbouring columns
+            both, size = inner, size // 2
+            inner = self._empty((pairs, size), x.dtype)
+            _check(self._elementwise.llmserve_gate_mul(
+                _pointer(both), _is_float(both), _pointer(inner), _is_float(inner), pairs, size, _ACTIVATIONS[activation], self._stream), "experts: gate")
         rows = self._empty((pairs, hidden), torch.float32)
         _check(library.llmserve_expert_product(
             _pointer(inner), _is_float(inner), _pointer(order), 0, _pointer(downs), hidden, size, _pointer(tiles), capacity, tile_rows, _pointer(rows),
             1, -1, self._stream), "experts: second product")
-        if shared is not None and (shared.dtype != torch.float32 or shared.shape != (tokens, hidden) or gates is None or gates.dtype != torch.float32):
+        if shared is not None and (shared.dtype != torch.float32 or shared.shape != (tokens, hidden) or (gates is not None and gates.dtype != torch.float32)):
             raise KernelError("experts: the shared rows and their gates are float32")
         out = self._empty((tokens, hidden), torch.float32)
         _check(library.llmserve_combine_pairs(
             _pointer(rows), _pointer(place), _pointer(weights), top, _pointer(out), tokens, hidden, _pointer(shared),
-            _pointer(gates if shared is not None else None), gates.shape[1] if shared is not None else 1, gate_column, self._stream), "experts: sum")
+            _pointer(gates if shared is not None else None), gates.shape[1] if shared is not None and gates is not None else 1, gate_column,
+            self._stream), "experts: sum")
         return out
 
     # ------------------------------------------------------------------ the gated delta rule
 
-    def causal_conv(self, x, channels: int, taps, activation: str, batch, window) -> torch.Tensor:
-        if activation != "silu":
+    def causal_conv(self, x, channels: int, taps, activation: str, batch, window, bias=None) -> torch.Tensor:
+        if activation not in ("silu", "none"):
             raise KernelError(f"causal_conv: no kernel applies {activation!r} behind the convolution")
+        if bias is not None and (bias.dtype != torch.float32 or bias.shape != (channels,)):
+            raise KernelError("causal_conv: a float32 bias a channel")
         tokens = x.shape[0]
         if taps.dtype != torch.float32 or taps.shape[0] != channels:
             raise KernelError("causal_conv: float32 taps, a row a channel")
@@ -1251,33 +1269,43 @@ class HipKernels:
         status = self._library_of("delta_rule").llmserve_causal_conv(
             _pointer(x), _is_float(x), tokens, x.shape[1], channels, _pointer(taps), width, _pointer(batch.token_sequence),
             _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], _pointer(window if width > 1 else None),
-            _pointer(out), self._stream,
+            _pointer(out), _pointer(bias), 1 if activation == "none" else 0, self._stream,
         )
         _check(status, "causal_conv")
         return out
 
-    def gated_delta_rule(self, mixed, controls, rate, step_bias, heads: int, kv_heads: int, dim: int, vdim: int, batch, state) -> torch.Tensor:
+    def _channel_steps(self, steps, controls, step_bias, tokens: int, heads: int, dim: int) -> None:
+        """Checks the operands of a decay per key channel: `steps` float32 [T, >= heads * dim], controls [T, heads] (b alone)."""
+        if steps.dtype != torch.float32 or steps.ndim != 2 or steps.shape[0] != tokens or steps.shape[1] < heads * dim:
+            raise KernelError("delta rule: the channels' steps are float32 [T, heads * dim (or more)]")
+        if controls.shape != (tokens, heads) or controls.dtype != torch.float32 or step_bias.shape != (heads * dim,):
+            raise KernelError("delta rule: with a decay per channel, float32 controls [b] and a bias a head and channel")
+
+    def gated_delta_rule(self, mixed, controls, rate, step_bias, heads: int, kv_heads: int, dim: int, vdim: int, batch, state,
+                         channel_steps=None) -> torch.Tensor:
         tokens = mixed.shape[0]
-        if mixed.shape[1] != 2 * kv_heads * dim + heads * vdim or controls.shape != (tokens, 2 * heads) or controls.dtype != torch.float32:
+        if channel_steps is not None:
+            self._channel_steps(channel_steps, controls, step_bias, tokens, heads, dim)
+        if mixed.shape[1] != 2 * kv_heads * dim + heads * vdim or controls.dtype != torch.float32 or (channel_steps is None and controls.shape != (tokens, 2 * heads)):
             raise KernelError("gated_delta_rule: rows of [q | k | v] and float32 controls [b | a]")
         if state.dtype != torch.float32 or state.shape[1:] != (heads, vdim, dim) or rate.dtype != torch.float32 or step_bias.dtype != torch.float32:
             raise KernelError("gated_delta_rule: the state is float32 [slots, heads, vdim, dim] (S transposed)")
         library = self._library_of("delta_rule")
         out = self._empty((tokens, heads * vdim), torch.float32)
         line = library.llmserve_delta_line(dim)
-        unit = self._empty((tokens, kv_heads, 2, line), torch.float32)  # unit k and q as the recurrence reads them
+        unit = self._empty((tokens, kv_heads, 2, line) if channel_steps is None else (tokens, heads, 3, line), torch.float32)  # unit k and q as the recurrence reads them
         gates = self._empty((tokens, heads, 2), torch.float32)  # decay and beta
         status = library.llmserve_gated_delta_rule(
             _pointer(mixed), _is_float(mixed), _pointer(controls), _pointer(rate), _pointer(step_bias), heads, kv_heads, dim, vdim,
             _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], tokens, int(getattr(batch, "max_query_length", tokens)),
             _pointer(unit), _pointer(gates),
-            _pointer(state), _pointer(out), self._stream,
+            _pointer(state), _pointer(out), _pointer(channel_steps), channel_steps.shape[1] if channel_steps is not None else 0, self._stream,
         )
         _check(status, "gated_delta_rule")
         return out
 
     def conv_gated_delta_rule(self, projected, channels: int, taps, activation: str, controls, rate, step_bias, heads: int, kv_heads: int,
-                              dim: int, vdim: int, batch, window, state) -> torch.Tensor:
+                              dim: int, vdim: int, batch, window, state, channel_steps=None) -> torch.Tensor:
         """`causal_conv` and `gated_delta_rule` in two kernels: one, parallel over tokens, convolves, makes the unit vectors
         and the gates; the other walks the tokens and moves the kept inputs on.  What lies between stays float32."""
         if activation != "silu":
@@ -1285,17 +1313,19 @@ class HipKernels:
         tokens, width = projected.shape[0], taps.shape[1]
         if channels > 12288:  # (more than the first kernel keeps in LDS)
             mixed = self.causal_conv(projected, channels, taps, activation, batch, window)
-            return self.gated_delta_rule(mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state)
+            return self.gated_delta_rule(mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state, channel_steps=channel_steps)
+        if channel_steps is not None:
+            self._channel_steps(channel_steps, controls, step_bias, tokens, heads, dim)
         if channels != 2 * kv_heads * dim + heads * vdim or taps.dtype != torch.float32 or taps.shape[0] != channels:
             raise KernelError("conv_gated_delta_rule: the convolutions run over [q | k | v], float32 taps a channel")
         if width > 1 and (window is None or window.dtype != torch.float32 or window.shape[1:] != (width - 1, channels)):
             raise KernelError("conv_gated_delta_rule: the kept inputs are float32 [slots, taps - 1, channels]")
-        if controls.shape != (tokens, 2 * heads) or controls.dtype != torch.float32 or state.dtype != torch.float32 or state.shape[1:] != (heads, vdim, dim):
+        if (channel_steps is None and controls.shape != (tokens, 2 * heads)) or controls.dtype != torch.float32 or state.dtype != torch.float32 or state.shape[1:] != (heads, vdim, dim):
             raise KernelError("conv_gated_delta_rule: float32 controls [b | a] and a float32 state [slots, heads, vdim, dim]")
         library = self._library_of("delta_rule")
         out = self._empty((tokens, heads * vdim), torch.float32)
         line = library.llmserve_delta_line(dim)
-        unit = self._empty((tokens, kv_heads, 2, line), torch.float32)
+        unit = self._empty((tokens, kv_heads, 2, line) if channel_steps is None else (tokens, heads, 3, line), torch.float32)
         gates = self._empty((tokens, heads, 2), torch.float32)
         values = self._empty((tokens, heads * vdim), torch.float32)
         status = library.llmserve_conv_gated_delta_rule(
@@ -1303,7 +1333,7 @@ class HipKernels:
             _pointer(window if width > 1 else None), _pointer(controls), _pointer(rate), _pointer(step_bias), heads, kv_heads, dim, vdim,
             _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], tokens,
             int(getattr(batch, "max_query_length", tokens)), _pointer(unit), _pointer(gates), _pointer(values), _pointer(state), _pointer(out),
-            self._stream,
+            _pointer(channel_steps), channel_steps.shape[1] if channel_steps is not None else 0, self._stream,
         )
         _check(status, "conv_gated_delta_rule")
         return out
@@ -1314,10 +1344,10 @@ class HipKernels:
         tokens = read.shape[0]
         if read.dtype != torch.float32 or read.shape[1] != heads * vdim or weight.shape != (vdim,):
             raise KernelError("gated_head_norm: a float32 read-out [T, heads * vdim] and a weight of vdim")
-        out = self._empty((tokens, heads * vdim), gates.dtype)
+        out = self._empty((tokens, heads * vdim), self.dtype)  # (gates that a product left in float32 gate a result in the run dtype)
         status = self._library_of("delta_rule").llmserve_gated_head_norm(
             _pointer(read), _pointer(gates), _is_float(gates), gates.shape[1], gate_first, _pointer(weight), _is_float(weight), eps,
-            tokens, heads, vdim, 1 if activation == "sigmoid" else 0, _pointer(out), self._stream,
+            tokens, heads, vdim, 1 if activation == "sigmoid" else 0, _is_float(out), _pointer(out), self._stream,
         )
         _check(status, "gated_head_norm")
         return out
@@ -1348,7 +1378,7 @@ class HipKernels:
 
     def assemble_heads(self, x, q_first: int, k_first: int, v_first: int, heads: int, kv_heads: int, dim: int, vdim: int, width: int,
                        norm, q_weight, k_weight, eps: float, table, rot_dims: int, other=None, other_first: int = 0, blend: float = 0.0,
-                       batch=None, cell=None):
+                       batch=None, cell=None, pairing: str = "adjacent"):
         """With a writable `cell` the keys and values are also stored in its pages: by this kernel in a step of single
         tokens, by the kernel that stores prompt portions (whole pieces of a page at a time) otherwise."""
         tokens = x.shape[0]
@@ -1375,7 +1405,7 @@ class HipKernels:
             _is_float(q_weight) if norm else 0, eps, _pointer(table if rot_dims else None), rot_dims, _pointer(other),
             other.shape[1] if other is not None else 0, other_first, float(blend), _pointer(out),
             _pointer(cell.keys if here else None), _pointer(cell.values if here else None), _pointer(group.slot_mapping if here else None),
-            group.page_size if here else 1, self._stream,
+            group.page_size if here else 1, _PAIRINGS[pairing], self._stream,
         )
         _check(status, "assemble_heads")
         if store and not here:
@@ -1431,6 +1461,69 @@ class HipKernels:
         return logits
 
     # ------------------------------------------------------------------ sampling
+
+    # ------------------------------------------------------------------ copies of the stream, a diagonal recurrence, weighted sums
+
+    def stream_copies(self, hidden, copies: int, scale: float) -> torch.Tensor:
+        tokens, width = hidden.shape
+        if hidden.dtype != torch.float32:
+            raise KernelError("stream_copies: the embedded rows are float32")
+        out = self._empty((tokens, copies * width), torch.float32)
+        status = self._library_of("streams").llmserve_stream_copies(_pointer(hidden), _pointer(out), tokens, width, copies, float(scale), self._stream)
+        _check(status, "stream_copies")
+        return out
+
+    def stream_norm(self, streams, pending, read, weight, eps: float, rows=None) -> torch.Tensor:
+        tokens, copies = streams.shape[0], read.shape[0]
+        width = streams.shape[1] // copies
+        if streams.dtype != torch.float32 or streams.shape[1] != copies * width or read.dtype != torch.float32 or weight.shape != (width,):
+            raise KernelError("stream_norm: float32 copies side by side, a float32 weight a copy, a norm weight as long as one copy")
+        result = mix = write = None
+        parts = 1
+        if pending is not None:
+            result, mix, write = pending.result, pending.mix, pending.out
+            parts = 1 if result.ndim == 2 else result.shape[0]
+            if result.dtype != torch.float32 or result.shape[-2:] != (tokens, width) or mix.shape != (copies, copies) or write.shape != (copies,) \
+                    or mix.dtype != torch.float32 or write.dtype != torch.float32:
+                raise KernelError("stream_norm: the pending result is float32 [(parts,) T, width], its weights float32 [copies, copies] and [copies]")
+        count = tokens if rows is None else rows.shape[0]
+        out = self._empty((count, width), self.dtype)
+        status = self._library_of("streams").llmserve_stream_norm(
+            _pointer(streams), _pointer(result), parts, tokens, _pointer(mix), _pointer(write), _pointer(read), _pointer(weight),
+            _is_float(weight), _pointer(out), _is_float(out), _pointer(rows), count, width, copies, eps, self._stream,
+        )
+        _check(status, "stream_norm")
+        return out
+
+    def add_scaled(self, a, a_scale: float, b, b_scale: float) -> torch.Tensor:
+        if a.dtype != torch.float32 or (b is not None and (b.dtype != torch.float32 or b.shape[-2:] != a.shape[-2:])):
+            raise KernelError("add_scaled: float32 results of one shape (or partial sums of them)")
+        rows, width = a.shape[-2:]
+        out = self._empty((rows, width), torch.float32)
+        status = self._library_of("streams").llmserve_add_scaled(
+            _pointer(a), 1 if a.ndim == 2 else a.shape[0], float(a_scale), _pointer(b), 1 if b is None or b.ndim == 2 else b.shape[0],
+            float(b_scale), _pointer(out), rows, width, self._stream,
+        )
+        _check(status, "add_scaled")
+        return out
+
+    def gated_recurrence(self, u, gates, gate_bias, rates, branch, branch_first: int, activation: str, blocks: int, batch, state) -> torch.Tensor:
+        if activation != "gelu_tanh":
+            raise KernelError(f"gated_recurrence: no kernel applies {activation!r} to the branch beside the recurrence")
+        tokens, width = u.shape
+        if gates.shape != (tokens, 2 * width) or gates.dtype != u.dtype or branch.dtype != u.dtype or branch.shape[0] != tokens:
+            raise KernelError("gated_recurrence: the gates' products are [T, 2 width] and the branch rows of the same type")
+        if gate_bias.dtype != torch.float32 or gate_bias.numel() != 2 * width or rates.dtype != torch.float32 or rates.shape != (width,) \
+                or state.dtype != torch.float32 or state.shape[1:] != (width,):
+            raise KernelError("gated_recurrence: float32 biases [blocks, 2 part], rates [width] and state [slots, width]")
+        out = self._empty((tokens, width), u.dtype)
+        status = self._library_of("recurrence").llmserve_gated_recurrence(
+            _pointer(u), _is_float(u), _pointer(gates), _pointer(gate_bias), _pointer(rates), _pointer(branch), branch.shape[1], branch_first,
+            width, blocks, _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0],
+            int(getattr(batch, "max_query_length", tokens)), _pointer(state), _pointer(out), self._stream,
+        )
+        _check(status, "gated_recurrence")
+        return out
 
     def _sampling_library(self):
         if self._sampling is None:

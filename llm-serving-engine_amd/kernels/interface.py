@@ -121,23 +121,29 @@ class Kernels(Protocol):
 
     # ------------------------------------------------------------------ the gated delta rule
 
-    def causal_conv(self, x: torch.Tensor, channels: int, taps: torch.Tensor, activation: str, batch: Any, window: torch.Tensor | None) -> torch.Tensor:
-        """act of the causal convolution per channel over each request's tokens, of the first `channels` columns of x;
-        taps float32 [channels, width], the last column the current token's.  `window` float32 [slots, width - 1,
+    def causal_conv(
+        self, x: torch.Tensor, channels: int, taps: torch.Tensor, activation: str, batch: Any, window: torch.Tensor | None,
+        bias: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """act (silu, or "none") of the causal convolution per channel (plus `bias`, float32 [channels]) over each request's
+        tokens, of the first `channels` columns of x; taps float32 [channels, width], the last column the current token's.  `window` float32 [slots, width - 1,
         channels] holds each request's last inputs (zeros at its start) and is moved on."""
 
     def gated_delta_rule(
         self, mixed: torch.Tensor, controls: torch.Tensor, rate: torch.Tensor, step_bias: torch.Tensor, heads: int,
-        kv_heads: int, dim: int, vdim: int, batch: Any, state: torch.Tensor,
+        kv_heads: int, dim: int, vdim: int, batch: Any, state: torch.Tensor, channel_steps: torch.Tensor | None = None,
     ) -> torch.Tensor:
-        """mixed [T, q | k | v], controls float32 [T, b | a]; q, k to unit length (q times dim^-1/2), beta = sigmoid(b),
+        """With `channel_steps` (float32 [T, heads * dim or more columns]) the decay is one a head and key channel,
+        g = exp(-exp(rate_h) softplus(channel_steps + step_bias)) with step_bias [heads * dim], row r of S scaled by g[r], and
+        controls is [T, b] alone.  Otherwise:
+        mixed [T, q | k | v], controls float32 [T, b | a]; q, k to unit length (q times dim^-1/2), beta = sigmoid(b),
         g = exp(-exp(rate) softplus(a + step_bias)); per request and head, token by token: S = g S; u = beta (v - S^T k);
         S += k u^T; o = S^T q.  `state` float32 [slots, heads, vdim, dim] holds S^T and is updated.  -> float32 [T, heads * vdim]."""
 
     def conv_gated_delta_rule(
         self, projected: torch.Tensor, channels: int, taps: torch.Tensor, activation: str, controls: torch.Tensor,
         rate: torch.Tensor, step_bias: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, batch: Any,
-        window: torch.Tensor | None, state: torch.Tensor,
+        window: torch.Tensor | None, state: torch.Tensor, channel_steps: torch.Tensor | None = None,
     ) -> torch.Tensor:
         """`causal_conv` followed by `gated_delta_rule` (a library may fuse them and keep what lies between in float32)."""
 
@@ -146,7 +152,7 @@ class Kernels(Protocol):
         vdim: int, activation: str,
     ) -> torch.Tensor:
         """Per head: read / rms(read) * weight * act(gates[:, gate_first + h * vdim : + vdim]) -> run dtype [T, heads * vdim];
-        act silu or sigmoid; weight of vdim for every head."""
+        act silu or sigmoid; weight of vdim for every head; the gates in the run dtype or float32."""
 
     # ------------------------------------------------------------------ norms on results, heads put together, linear attention
 
@@ -161,13 +167,14 @@ class Kernels(Protocol):
         self, x: torch.Tensor, q_first: int, k_first: int, v_first: int, heads: int, kv_heads: int, dim: int, vdim: int,
         width: int, norm: str | None, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
         table: torch.Tensor | None, rot_dims: int, other: torch.Tensor | None = None, other_first: int = 0, blend: float = 0.0,
-        batch: Any = None, cell: Any = None,
+        batch: Any = None, cell: Any = None, pairing: str = "adjacent",
     ) -> torch.Tensor:
         """From rows that hold `heads` queries and `kv_heads` keys of `dim` and `kv_heads` values of `vdim` (from the
         columns q_first, k_first, v_first): rows [T, (heads + 2 kv_heads) * width] of queries, keys and values of
         `width`, zeros beyond a head's own size.  Queries and keys are RMS-normed (`norm` "head": every head by
         itself, weights of dim; "row": all query heads together and all key heads together, weights as long as
-        they; None), then their first `rot_dims` dimensions turned in adjacent pairs by the token's row of `table`
+        they; None), then their first `rot_dims` dimensions turned in pairs (`pairing` "adjacent": (2i, 2i + 1); "half":
+        (i, i + rot_dims / 2)) by the token's row of `table`
         (float32 [T, rot_dims / 2, 2], cos and sin).  With `other`: v <- (1 - blend) v + blend * other[:, other_first : + kv_heads * vdim].
         With a writable `cell` (and the step's `batch`) the keys and values are also stored in the cell's pages, as
         `rotate_and_store` without a rotation would store them."""
@@ -188,18 +195,49 @@ class Kernels(Protocol):
 
     # ------------------------------------------------------------------ routed experts
 
-    def route(self, scores: torch.Tensor, experts: int, correction: torch.Tensor, top: int, scale: float, scoring: str):
-        """s = squash(scores[:, :experts]); the `top` largest of s + correction choose (the lower index among equals);
-        -> (int32 [T, top] experts, float32 [T, top] weights = scale * s of the chosen)."""
+    def route(
+        self, scores: torch.Tensor, experts: int, correction: torch.Tensor | None, top: int, scale: float, scoring: str,
+        groups: int = 1, keep_groups: int = 1, renormalise: bool = False,
+    ):
+        """s = squash(scores[:, :experts]) (sigmoid of each, or softmax over all); the `top` largest of s + correction (None:
+        of s) choose (the lower index among equals), among the experts of the `keep_groups` best of `groups` equal groups of
+        neighbours (a group's score is its largest); -> (int32 [T, top] experts, float32 [T, top] weights = scale * s of the
+        chosen, with `renormalise` scale * s / (sum of the chosen s + 1e-20))."""
 
-    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str) -> Any: ...
+    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str, gates: list[torch.Tensor] | None = None) -> Any:
+        """With `gates` an expert is down(act(gate x) * (up x)), else down(act(up x))."""
 
     def expert_feed_forward(
         self, x: torch.Tensor, experts: Any, chosen: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None = None,
         gates: torch.Tensor | None = None, gate_column: int = 0,
     ) -> torch.Tensor:
-        """sum over a token's chosen experts of weight * down_e(act(up_e x)) (+ sigmoid(gates[:, gate_column]) * shared),
-        float32 [T, hidden]; the inner rows are rounded to the run dtype between the two products."""
+        """sum over a token's chosen experts of weight * down_e(act(up_e x)) (+ sigmoid(gates[:, gate_column]) * shared, or
+        + shared where no gates are given), float32 [T, hidden]; the inner rows are rounded to the run dtype between the
+        two products."""
+
+    # ------------------------------------------------------------------ copies of the stream, a diagonal recurrence, weighted sums
+
+    def stream_copies(self, hidden: torch.Tensor, copies: int, scale: float) -> torch.Tensor:
+        """float32 [T, copies * width]: the rows times `scale`, `copies` times side by side."""
+
+    def stream_norm(
+        self, streams: torch.Tensor, pending: Any, read: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """`streams` float32 [T, copies * width].  With `pending` (`.result` float32 [T, width] or partial sums of it, `.mix`
+        float32 [copies, copies] from -> to, `.out` float32 [copies]): x_t <- sum_s mix[s, t] x_s + out[t] * result, in place.
+        Then u = sum_s read[s] x_s and u * rsqrt(mean(u^2) + eps) * weight in the run dtype.  With `rows` (int32 token rows)
+        only those rows are computed and returned, and the copies stay as they are."""
+
+    def gated_recurrence(
+        self, u: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor, rates: torch.Tensor, branch: torch.Tensor, branch_first: int,
+        activation: str, blocks: int, batch: Any, state: torch.Tensor,
+    ) -> torch.Tensor:
+        """u [T, width]; gates [T, blocks * (r part | i part)] before their bias (float32, the same layout) and sigmoid;
+        a = exp(rates * r); per request, token by token: S <- a S + sqrt(1 - a^2) i u; -> S * act(branch[:, branch_first : +
+        width]) in the run dtype.  `state` float32 [slots, width] holds S and is updated."""
+
+    def add_scaled(self, a: torch.Tensor, a_scale: float, b: torch.Tensor | None, b_scale: float) -> torch.Tensor:
+        """float32 [T, width]: a_scale * a + b_scale * b, where a and b are float32 results or partial sums [parts, T, width]."""
 
     def gather_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
         """float32 (hidden + delta)[rows]."""

@@ -15,6 +15,8 @@ DEFAULT_VARIANTS: dict[str, list[dict[str, object]]] = {
     "gemm_rows": [{}],
     "delta_rule": [{}],
     "heads": [{}],
+    "streams": [{}],
+    "recurrence": [{}],
     # query/key sizes of the tests' and the benchmark's models with decaying linear attention
     "decay_attention": [{"HEAD_DIM": d} for d in (8, 16, 24, 32, 48, 64, 128)],
     # head sizes of the tests' models and kernel tests, and of the benchmark
