@@ -33,6 +33,11 @@ same width, number of layer runs and vocabulary: decoding at --batch and the pre
     python bench.py --op sozavik
 
 does the same for the third (configs/sozavik-w1536.json, configs/sozavik-w3584.json).
+
+    python bench.py --op katenex
+
+measures the fourth (configs/katenex-w1536.json, configs/katenex-w3584.json) beside the Dafutar models of the same width
+and number of layer runs (the engine's other decoder with the delta rule and routed experts) and the Qwen2 models.
 """
 
 from __future__ import annotations
@@ -74,7 +79,7 @@ def parse() -> argparse.Namespace:
                         help="leave out decoding at contexts of 8k and 30k (batch 8) and 4k (batch 64), and the long prompts")
     parser.add_argument("--skip-other-models", action="store_true",
                         help="leave out the float32 run and the 7B and 32B layer sizes")
-    parser.add_argument("--op", choices=("decode-attention", "prefill-attention", "dafutar", "sozavik"), default=None,
+    parser.add_argument("--op", choices=("decode-attention", "prefill-attention", "dafutar", "sozavik", "katenex"), default=None,
                         help="measure one operation alone instead, as the reference's kernel benchmark does")
     return parser.parse_args()
 
@@ -427,6 +432,8 @@ def main() -> int:
         return dafutar_table(args)
     if args.op == "sozavik":
         return sozavik_table(args)
+    if args.op == "katenex":
+        return katenex_table(args)
 
     import torch
 
@@ -570,18 +577,27 @@ def sozavik_table(args) -> int:
     return beside_qwen2(args, "sozavik", "Sozavik")
 
 
-def beside_qwen2(args, name: str, title: str) -> int:
+def katenex_table(args) -> int:
+    """The Katenex decoder (several copies of the stream; layers of the delta rule with a decay per key channel and of
+    softmax attention beside a gated linear recurrence; experts chosen within groups) at two layer sizes beside the
+    Dafutar and the Qwen2 of the same width, number of layer runs and vocabulary, measured as `dafutar_table` measures."""
+    return beside_qwen2(args, "katenex", "Katenex", also=("dafutar",))
+
+
+def beside_qwen2(args, name: str, title: str, also: tuple[str, ...] = ()) -> int:
     import torch
 
     pairs = [
-        ("w1536", ROOT / "configs" / f"{name}-w1536.json", ROOT / "configs" / "qwen2-w1536-12-layers.json"),
-        ("w3584", ROOT / "configs" / f"{name}-w3584.json", ROOT / "configs" / "qwen2-w3584-4-layers.json"),
+        ("w1536", ROOT / "configs" / f"{name}-w1536.json", *(ROOT / "configs" / f"{other}-w1536.json" for other in also),
+         ROOT / "configs" / "qwen2-w1536-12-layers.json"),
+        ("w3584", ROOT / "configs" / f"{name}-w3584.json", *(ROOT / "configs" / f"{other}-w3584.json" for other in also),
+         ROOT / "configs" / "qwen2-w3584-4-layers.json"),
     ]
     steps, warmup, repeats = max(1, min(args.steps, 64)), min(args.warmup, 8), min(max(1, args.repeats), 3)
     shape = (args.batch, args.prompt_len, output_tokens(args.batch, args.prompt_len, steps, warmup))
     points: dict = {}
     for tag, *paths in pairs:
-        for label, path in zip((name, "qwen2"), paths):
+        for label, path in zip((name, *also, "qwen2"), paths):
             bench = Bench(str(path), args.dtype, args.seed, library_products=not args.own_products, shapes=[shape], prefill_tokens=args.prefill_len)
             decode = bench.decode(args.batch, args.prompt_len, steps, warmup, repeats)
             prefill = bench.prefill(args.prefill_len, repeats=3)
@@ -596,7 +612,8 @@ def beside_qwen2(args, name: str, title: str) -> int:
             del bench
             torch.cuda.empty_cache()
     print(json.dumps({
-        "metric": f"decode tok/s at batch {args.batch} and prefill tok/s of {args.prefill_len} tokens, {title} beside Qwen2 at equal sizes",
+        "metric": f"decode tok/s at batch {args.batch} and prefill tok/s of {args.prefill_len} tokens, {title} beside "
+                  f"{' and '.join(other.capitalize() for other in (*also, 'qwen2'))} at equal sizes",
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": args.dtype,
         "data": "synthetic: seeded random weights, uniform random token ids", "points": points,
     }))

@@ -4,22 +4,24 @@
 // where the gates' columns come in `blocks` parts of the channels, a part's r columns before its i columns.  Gates,
 // decays and S are float32; u, the gates' products and the branch come in bfloat16 or float32.
 //
-// The state of a channel meets no other channel.  A workgroup owns 64 channels of one request; a long portion is cut
+// The state of a channel meets no other channel.  A workgroup owns CH channels of one request; a long portion is cut
 // into as many runs of tokens as the workgroup has rows of threads: every row first walks its run from an empty state and
 // notes the product of its decays and what it ends with, then takes the state that the runs before it leave
 // (S_end = A S_in + B, run after run) and walks its run again for the results.  The last row leaves the request's state.
+// The walk is a chain of dependent steps, each with four exponentials, so its length is what counts: a portion of
+// hundreds of tokens goes to workgroups of 16 channels and 64 runs (a run of a 2,048-token prompt is 32 tokens), a step
+// of single tokens to workgroups of 64 channels and one run.
 #include "common.h"
 
-#define CHANNELS 64
-#define MAX_RUNS 16
+#define MAX_THREADS 1024
 
-template <typename T>
-__global__ __launch_bounds__(CHANNELS * MAX_RUNS) void gated_recurrence_kernel(
+template <typename T, int CH>
+__global__ __launch_bounds__(MAX_THREADS) void gated_recurrence_kernel(
     const T* __restrict__ u, const T* __restrict__ gates, const float* __restrict__ bias, const float* __restrict__ rates,
     const T* __restrict__ branch, int branch_stride, int branch_first, int width, int part, const int* __restrict__ start,
     const int* __restrict__ slots, float* __restrict__ state, T* __restrict__ out) {
-  __shared__ float decays[MAX_RUNS][CHANNELS], ends[MAX_RUNS][CHANNELS];
-  const int b = blockIdx.x, c = blockIdx.y * CHANNELS + threadIdx.x, run = threadIdx.y, runs = blockDim.y;
+  __shared__ float decays[MAX_THREADS / CH][CH], ends[MAX_THREADS / CH][CH];
+  const int b = blockIdx.x, c = blockIdx.y * CH + threadIdx.x, run = threadIdx.y, runs = blockDim.y;
   const int first = start[b], count = start[b + 1] - first;
   if (count <= 0) return;
   const bool owns = c < width;
@@ -69,13 +71,19 @@ extern "C" int llmserve_gated_recurrence(const void* u, int is_float, const void
                                          hipStream_t stream) {
   if (requests <= 0) return 0;
   if (width < 1 || blocks < 1 || width % blocks || branch_first < 0 || branch_first + width > branch_stride) return ERR_BAD_ARGUMENT;
-  const int runs = longest <= 8 ? 1 : longest <= 64 ? 4 : MAX_RUNS;
-  const dim3 grid(requests, (width + CHANNELS - 1) / CHANNELS), block(CHANNELS, runs);
-  if (is_float)
-    hipLaunchKernelGGL(gated_recurrence_kernel<float>, grid, block, 0, stream, (const float*)u, (const float*)gates, bias, rates,
-                       (const float*)branch, branch_stride, branch_first, width, width / blocks, start, slots, state, (float*)out);
-  else
-    hipLaunchKernelGGL(gated_recurrence_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)u, (const bf16_t*)gates, bias, rates,
-                       (const bf16_t*)branch, branch_stride, branch_first, width, width / blocks, start, slots, state, (bf16_t*)out);
+#define LAUNCH_RECURRENCE(T, CH, RUNS)                                                                                            \
+  hipLaunchKernelGGL((gated_recurrence_kernel<T, CH>), dim3(requests, (width + CH - 1) / CH), dim3(CH, RUNS), 0, stream, (const T*)u, \
+                     (const T*)gates, bias, rates, (const T*)branch, branch_stride, branch_first, width, width / blocks, start,     \
+                     slots, state, (T*)out)
+#define LAUNCH_RECURRENCE_BY_LENGTH(T)                                                         \
+  do {                                                                                         \
+    if (longest <= 8) LAUNCH_RECURRENCE(T, 64, 1);                                             \
+    else if (longest <= 64) LAUNCH_RECURRENCE(T, 64, 4);                                       \
+    else if (longest <= 256) LAUNCH_RECURRENCE(T, 32, 16);                                     \
+    else LAUNCH_RECURRENCE(T, 16, 64);                                                         \
+  } while (0)
+  if (is_float) LAUNCH_RECURRENCE_BY_LENGTH(float); else LAUNCH_RECURRENCE_BY_LENGTH(bf16_t);
+#undef LAUNCH_RECURRENCE_BY_LENGTH
+#undef LAUNCH_RECURRENCE
   return LAUNCH_STATUS();
 }

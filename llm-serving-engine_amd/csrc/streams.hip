@@ -25,14 +25,17 @@ extern "C" int llmserve_stream_copies(const float* hidden, float* out, int token
 // One workgroup a row.  With `result` (float32 [parts, tokens, width], its parts added in order): the copies of the row
 // become x_t <- sum_s mix[s, t] x_s + write[t] * result, all from the old ones, and go back to memory unless `rows` picks
 // the rows (then the copies stay as they are: nobody reads them again).  Then u = sum_s read[s] x_s, and
-// out = u * rsqrt(mean(u^2) + eps) * weight.  Everything float32; `out` in the run's type.
-template <typename TO>
-__global__ __launch_bounds__(256) void stream_norm_kernel(float* __restrict__ streams, const float* __restrict__ result, int parts,
-                                                          size_t part_stride, const float* __restrict__ mix, const float* __restrict__ write,
-                                                          const float* __restrict__ read, const void* __restrict__ weight, int weight_is_float,
-                                                          TO* __restrict__ out, const int* __restrict__ rows, int width, int copies, float eps) {
+// out = u * rsqrt(mean(u^2) + eps) * weight.  Everything float32; `out` in the run's type.  A thread takes V neighbouring
+// columns at a time (V = 4 where the width allows 16-byte loads), so a row of a few thousand columns is one pass of
+// loads that are all in flight together: a step of few rows is as long as its longest workgroup.
+template <typename TO, int V>
+__global__ __launch_bounds__(1024) void stream_norm_kernel(float* __restrict__ streams, const float* __restrict__ result, int parts,
+                                                           size_t part_stride, const float* __restrict__ mix, const float* __restrict__ write,
+                                                           const float* __restrict__ read, const void* __restrict__ weight, int weight_is_float,
+                                                           TO* __restrict__ out, const int* __restrict__ rows, int width, int copies, float eps) {
   extern __shared__ float summed[];  // [width]: u
   __shared__ float shared[17];
+  struct alignas(sizeof(float) * V) Piece { float v[V]; };
   const size_t t = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
   float* mine = streams + t * copies * width;
   float links[MAX_COPIES][MAX_COPIES], outward[MAX_COPIES], inward[MAX_COPIES];
@@ -44,31 +47,55 @@ __global__ __launch_bounds__(256) void stream_norm_kernel(float* __restrict__ st
     for (int d = 0; d < MAX_COPIES; ++d) links[s][d] = (result && s < copies && d < copies) ? mix[s * copies + d] : 0.f;
   }
   float squares = 0.f;
-  for (int h = threadIdx.x; h < width; h += blockDim.x) {
-    float x[MAX_COPIES];
+  for (int h = threadIdx.x * V; h < width; h += blockDim.x * V) {
+    Piece x[MAX_COPIES];
 #pragma unroll
-    for (int s = 0; s < MAX_COPIES; ++s) x[s] = s < copies ? mine[(size_t)s * width + h] : 0.f;
-    float u = 0.f;
+    for (int s = 0; s < MAX_COPIES; ++s) {
+      if (s < copies) {
+        x[s] = *(const Piece*)(mine + (size_t)s * width + h);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) x[s].v[j] = 0.f;
+      }
+    }
+    Piece u;
+#pragma unroll
+    for (int j = 0; j < V; ++j) u.v[j] = 0.f;
     if (result) {
-      float y = 0.f;
-      for (int p = 0; p < parts; ++p) y += result[p * part_stride + t * width + h];
+      Piece y;
+#pragma unroll
+      for (int j = 0; j < V; ++j) y.v[j] = 0.f;
+      for (int p = 0; p < parts; ++p) {
+        const Piece part = *(const Piece*)(result + p * part_stride + t * width + h);
+#pragma unroll
+        for (int j = 0; j < V; ++j) y.v[j] += part.v[j];
+      }
 #pragma unroll
       for (int d = 0; d < MAX_COPIES; ++d) {
         if (d < copies) {
-          float fresh = 0.f;
+          Piece fresh;
 #pragma unroll
-          for (int s = 0; s < MAX_COPIES; ++s) fresh += links[s][d] * x[s];
-          fresh += outward[d] * y;
-          if (!rows) mine[(size_t)d * width + h] = fresh;
-          u += inward[d] * fresh;
+          for (int j = 0; j < V; ++j) {
+            float sum = 0.f;
+#pragma unroll
+            for (int s = 0; s < MAX_COPIES; ++s) sum += links[s][d] * x[s].v[j];
+            fresh.v[j] = sum + outward[d] * y.v[j];
+            u.v[j] += inward[d] * fresh.v[j];
+          }
+          if (!rows) *(Piece*)(mine + (size_t)d * width + h) = fresh;
         }
       }
     } else {
 #pragma unroll
-      for (int s = 0; s < MAX_COPIES; ++s) u += inward[s] * x[s];
+      for (int s = 0; s < MAX_COPIES; ++s)
+#pragma unroll
+        for (int j = 0; j < V; ++j) u.v[j] += inward[s] * x[s].v[j];
     }
-    summed[h] = u;
-    squares += u * u;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      summed[h + j] = u.v[j];
+      squares += u.v[j] * u.v[j];
+    }
   }
   const float scale = rsqrtf(block_sum(squares, shared) / (float)width + eps);
   for (int h = threadIdx.x; h < width; h += blockDim.x)
@@ -81,13 +108,19 @@ extern "C" int llmserve_stream_norm(float* streams, const float* result, int par
   if (count <= 0) return 0;
   if (width < 1 || width > 16384 || copies < 1 || copies > MAX_COPIES || (result && (parts < 1 || !mix || !write))) return ERR_BAD_ARGUMENT;
   const size_t lds = (size_t)width * sizeof(float), part_stride = (size_t)tokens * width;
-  const int threads = width <= 64 ? 64 : width <= 128 ? 128 : 256;
-  if (out_is_float)
-    hipLaunchKernelGGL(stream_norm_kernel<float>, dim3(count), dim3(threads), lds, stream, streams, result, parts, part_stride, mix, write,
-                       read, weight, weight_is_float, (float*)out, rows, width, copies, eps);
-  else
-    hipLaunchKernelGGL(stream_norm_kernel<bf16_t>, dim3(count), dim3(threads), lds, stream, streams, result, parts, part_stride, mix, write,
-                       read, weight, weight_is_float, (bf16_t*)out, rows, width, copies, eps);
+  // 16-byte pieces where every copy of every row starts on a 16-byte border
+  const int pieces = width % 4 == 0 ? 4 : 1;
+  const int columns = width / pieces;
+  const int threads = columns <= 64 ? 64 : min(1024, WAVE * ((columns + WAVE - 1) / WAVE));
+#define LAUNCH_STREAM_NORM(TO, V)                                                                                                 \
+  hipLaunchKernelGGL((stream_norm_kernel<TO, V>), dim3(count), dim3(threads), lds, stream, streams, result, parts, part_stride, mix, \
+                     write, read, weight, weight_is_float, (TO*)out, rows, width, copies, eps)
+  if (out_is_float) {
+    if (pieces == 4) LAUNCH_STREAM_NORM(float, 4); else LAUNCH_STREAM_NORM(float, 1);
+  } else {
+    if (pieces == 4) LAUNCH_STREAM_NORM(bf16_t, 4); else LAUNCH_STREAM_NORM(bf16_t, 1);
+  }
+#undef LAUNCH_STREAM_NORM
   return LAUNCH_STATUS();
 }
 

@@ -1221,9 +1221,10 @@ class HipKernels:
         library = self._library_of("gemm_rows")
         pairs = tokens * top
         # tiles of 64 rows for the matrix cores where an expert has that many rows or so, else of 16
-        on_cores = x.dtype == torch.bfloat16 and hidden % 32 == 0 and size % 32 == 0
+        width = size // 2 if gated else size  # (the second product's inner size)
+        on_cores = x.dtype == torch.bfloat16 and hidden % 32 == 0 and width % 32 == 0
         tile_rows = 64 if on_cores and pairs >= 32 * count else 16
-        if on_cores and pairs >= 96 * count and hidden % 64 == 0 and size % 64 == 0:
+        if on_cores and pairs >= 96 * count and hidden % 64 == 0 and width % 64 == 0:
             tile_rows = 128  # many rows an expert: both operands through LDS
         capacity = -(-pairs // tile_rows) + count
         place = self._empty((pairs,), torch.int32)

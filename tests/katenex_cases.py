@@ -68,6 +68,19 @@ MIXED = config_of(
 )
 
 
+def with_every_expert(values: dict) -> dict:
+    """The same model with every expert of a layer used by every token (all groups kept): the router still weighs
+    them, but chooses nothing, so no rounding can turn a choice."""
+    values = json.loads(json.dumps(values))
+    for layer in values["layers"]:
+        if layer["mlp"] is not None:
+            router = layer["mlp"]["router"]
+            router["top"] = router["experts"]
+            if "groups" in router:
+                router["groups"]["keep"] = router["groups"]["count"]
+    return values
+
+
 def random_tensors(values: dict, seed: int, *, sharp: bool = False) -> dict[str, torch.Tensor]:
     """bfloat16 tensors by the model's own list of names and shapes.  Matrices are drawn so that activations stay
     of order one; norms, biases, decays and the links between the copies of the stream are far enough from one and

@@ -415,7 +415,7 @@ class TorchKernels:
         r = torch.sigmoid(z[..., :part]).reshape(tokens, width)
         i = torch.sigmoid(z[..., part:]).reshape(tokens, width)
         a = torch.exp(rates.float() * r)
-        push = torch.sqrt(1.0 - a * a) * i * u.float()
+        push = torch.sqrt(-torch.expm1(2.0 * rates.float() * r)) * i * u.float()  # sqrt(1 - a^2), exact also where a is near one
         y = torch.nn.functional.gelu(branch[:, branch_first : branch_first + width].float(), approximate="tanh")
         out = torch.zeros((tokens, width))
         row = 0
