@@ -144,7 +144,7 @@ class KatenexConfig(ArchitectureConfig):
 
     vocab: int
     width: int
-    streams: int
+    streams: int | None  # copies of the residual stream; None: one stream with the plain residual sum (no link tensors)
     embedding_scale: float
     norm_eps: float
     layers: tuple[KatenexLayer, ...]
@@ -196,7 +196,7 @@ class KatenexConfig(ArchitectureConfig):
             mixer = _read_mixer(kind, _mapping(entry.get("mixer"), f"{where}.mixer"), f"{where}.mixer")
             layers.append(KatenexLayer(kind, mixer, _read_mlp(entry.get("mlp"), f"{where}.mlp")))
         return cls(
-            vocab=reader.integer("vocab"), width=reader.integer("width"), streams=reader.integer("streams", default=1),
+            vocab=reader.integer("vocab"), width=reader.integer("width"), streams=reader.integer("streams", minimum=1) if values.get("streams") is not None else None,
             embedding_scale=embedding.number("scale", default=1.0), norm_eps=norm.number("eps"), layers=tuple(layers),
         )
 
@@ -246,5 +246,8 @@ class KatenexConfig(ArchitectureConfig):
                 if mlp.shared_ff is not None:
                     feed["shared"] = {"ff": mlp.shared_ff}
             layers.append({"type": layer.type, "mixer": described, "mlp": feed})
-        return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "streams": self.streams,
-                "embedding": {"scale": self.embedding_scale}, "norm": {"eps": self.norm_eps}, "layers": layers}
+        described = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width,
+                     "embedding": {"scale": self.embedding_scale}, "norm": {"eps": self.norm_eps}, "layers": layers}
+        if self.streams is not None:
+            described["streams"] = self.streams
+        return described

@@ -55,10 +55,12 @@ def _feed_forward_spec(config: KatenexConfig, mlp):
 
 def katenex_spec(config: KatenexConfig) -> ModelSpec:
     norm = RMSNormSpec(config.width, config.norm_eps, weight_name="")
+    copies, learned = (config.streams, True) if config.streams is not None else (1, False)
     layers, ignored = [], []
     for index, layer in enumerate(config.layers):
         feed_forward = _feed_forward_spec(config, layer.mlp)
-        block = HyperBlockSpec(config.streams, norm, _mixer_spec(config, layer.mixer), norm if feed_forward is not None else None, feed_forward)
+        block = HyperBlockSpec(copies, norm, _mixer_spec(config, layer.mixer), norm if feed_forward is not None else None, feed_forward,
+                               learned_links=learned)
         layers.append(LayerDefinition(f"l{index}.", block))
         if feed_forward is None:  # a folder may still hold what belongs to the feed-forward that is not there
             ignored += [f"l{index}.norm2", f"l{index}.hc2.in", f"l{index}.hc2.out", f"l{index}.hc2.mix"]
@@ -67,12 +69,12 @@ def katenex_spec(config: KatenexConfig) -> ModelSpec:
         hidden_size=config.width,
         layers=tuple(layers),
         run_order=tuple(LayerRun(index) for index in range(len(layers))),
-        final_norm=StreamNormSpec(config.width, config.norm_eps, config.streams, weight_name=""),
+        final_norm=StreamNormSpec(config.width, config.norm_eps, copies, weight_name=""),
         tie_embeddings=False,
         embedding_name="embed",
         final_norm_name="final.norm",
         head_name="head",
-        input_parts=(NamedPart("embedding.", StreamCopiesSpec(config.streams, config.embedding_scale)),),
+        input_parts=(NamedPart("embedding.", StreamCopiesSpec(copies, config.embedding_scale)),),
         ignored_tensors=tuple(ignored),
     )
 

@@ -110,6 +110,7 @@ class HyperBlockSpec:
     feed_forward_name: str = "mlp."
     mixer_links: str = "hc1."
     feed_forward_links: str = "hc2."
+    learned_links: bool = True  # False: no such tensors; every weight is one (one copy: the plain residual sum x <- x + y)
     kind: str = "hyper"
 
 
@@ -135,9 +136,10 @@ class HyperBlock(Block):
         found: dict[str, TensorSpec] = {}
         for name, registry, member in cls._members(spec):
             found.update(prefixed(registry.tensors(member), name))
-        found.update(prefixed(_links(spec.copies), spec.mixer_links))
-        if spec.feed_forward is not None:
-            found.update(prefixed(_links(spec.copies), spec.feed_forward_links))
+        if spec.learned_links:
+            found.update(prefixed(_links(spec.copies), spec.mixer_links))
+            if spec.feed_forward is not None:
+                found.update(prefixed(_links(spec.copies), spec.feed_forward_links))
         return found
 
     @classmethod
@@ -151,7 +153,12 @@ class HyperBlock(Block):
         self.feed_forward_norm, self.feed_forward = built[2:] if len(built) > 2 else (None, None)
         self.replayable = all(part.replayable for part in built)
 
+        if not spec.learned_links and spec.copies != 1:
+            raise ValueError("hyper block: several copies of the stream need their links")
+
         def links(prefix: str):
+            if not spec.learned_links:
+                return tuple(kernels.to_device(torch.ones(shape)) for shape in ((1,), (1, 1), (1,)))
             own = under(tensors, prefix)
             return tuple(kernels.to_device(own[name].float().contiguous()) for name in ("in", "mix", "out"))
 

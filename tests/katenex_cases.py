@@ -51,8 +51,11 @@ def moe(experts=6, top=2, scale=1.25, ff=12, shared=20, groups=(3, 2)):
 
 def config_of(layers, streams=3, vocab=67, width=32, eps=1e-5, scale=3.0):
     """`layers`: [(mixer entry, mlp or None)]."""
-    return {"architecture": "Katenex", "vocab": vocab, "width": width, "streams": streams, "embedding": {"scale": scale},
-            "norm": {"eps": eps}, "layers": [dict(mixer, mlp=mlp) for mixer, mlp in layers]}
+    found = {"architecture": "Katenex", "vocab": vocab, "width": width, "streams": streams, "embedding": {"scale": scale},
+             "norm": {"eps": eps}, "layers": [dict(mixer, mlp=mlp) for mixer, mlp in layers]}
+    if streams is None:  # the plain residual sum
+        del found["streams"]
+    return found
 
 
 # A model with both kinds of layer and sizes that differ wherever they can.

@@ -170,12 +170,15 @@ def forward(config, tensors, tokens):
     """-> (logits [T, vocab], the sum of the streams after every layer [layers, T, width])."""
     eps = config["norm"]["eps"]
     x = tensors["embed"][torch.as_tensor(tokens, dtype=torch.long)] * config["embedding"]["scale"]
-    streams = [x.clone() for _ in range(config["streams"])]
+    streams = [x.clone() for _ in range(config.get("streams") or 1)]
     count = len(streams)
     after = []
 
     def sublayer(name, norm, run):
         nonlocal streams
+        if config.get("streams") is None:  # one stream and the plain residual sum: x <- x + sublayer(norm(x))
+            streams = [streams[0] + run(rms_norm(streams[0], tensors[norm], eps))]
+            return
         read, write, mix = tensors[name + ".in"], tensors[name + ".out"], tensors[name + ".mix"]
         u = sum(read[s] * streams[s] for s in range(count))
         y = run(rms_norm(u, tensors[norm], eps))

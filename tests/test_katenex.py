@@ -53,6 +53,9 @@ def test_config_round_trip_and_refusals():
         target[path[-1]] = value
         with pytest.raises(ConfigError):
             KatenexConfig.from_dict(broken)
+    plain_sum = KatenexConfig.from_dict({key: value for key, value in cases.MIXED.items() if key != "streams"})
+    assert plain_sum.streams is None and "streams" not in plain_sum.to_config_json()
+    assert KatenexConfig.from_dict(plain_sum.to_config_json()) == plain_sum
     without = {key: value for key, value in cases.MIXED.items() if key != "width"}
     with pytest.raises(ConfigError, match="width"):
         KatenexConfig.from_dict(without)
@@ -105,6 +108,7 @@ ALONE = {
     "one expert a token, no groups": cases.config_of([(cases.parallel(), cases.moe(7, 1, 1.0, 8, 4, None))], streams=4),
     "all experts": cases.config_of([(cases.delta(conv=2), cases.moe(4, 4, 1.0, 8, 12, (4, 4)))]),
     "one copy of the stream": cases.config_of([(cases.delta(), cases.moe()), (cases.parallel(), cases.moe())], streams=1, scale=1.0),
+    "the plain residual sum": cases.config_of([(cases.delta(), cases.moe()), (cases.parallel(), None)], streams=None),
 }
 
 
@@ -114,7 +118,7 @@ def test_each_mechanism_layer_by_layer(tmp_path, name):
     tokens = cases.tokens_of(19, ALONE[name]["vocab"], seed=5)
     want_logits, want_streams = oracle(folder, tokens)
     runner = runner_for(folder)
-    copies = ALONE[name]["streams"]
+    copies = ALONE[name].get("streams") or 1
     seen = []
     runner.model.observer = lambda index, hidden, pending: seen.append(pending.applied(hidden).view(hidden.shape[0], copies, -1).sum(1).clone())
     logits = runner.step([StepEntry("a", tokens, range(len(tokens)))], create_missing=True)
