@@ -29,6 +29,32 @@ __device__ __forceinline__ float activation_of(int activation, float z) {
   }
 }
 
+// A code of ACT_GATED or more asks the matrix-core kernels of the experts for a gated result: the product's columns are
+// gates and ups in turn (gate_0, up_0, gate_1, ...), and column j of the result, half as wide, is act(gate_j) * up_j,
+// both rounded to the result's type first, as they would be if the product were stored and gated by a kernel behind it.
+#define ACT_GATED 16
+
+// A lane's four neighbouring columns n0 .. n0 + 3 (n0 a multiple of four) of a row of a product `outputs` wide.
+template <typename TO>
+__device__ __forceinline__ void store_four(TO* __restrict__ out, size_t row, int n0, int outputs, int activation, const f32x4& v) {
+  if (activation < ACT_GATED) {
+    TO* dst = out + row * outputs;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n0 + i < outputs) dst[n0 + i] = from_float<TO>(activation_of(activation, v[i]));
+    return;
+  }
+  TO* dst = out + row * (outputs / 2);
+#pragma unroll
+  for (int pair = 0; pair < 2; ++pair) {
+    const int n = n0 + 2 * pair;
+    if (n + 1 < outputs) {
+      const float gate = to_float(from_float<TO>(v[2 * pair])), up = to_float(from_float<TO>(v[2 * pair + 1]));
+      dst[n / 2] = from_float<TO>(activation_of(activation - ACT_GATED, gate) * up);
+    }
+  }
+}
+
 // Thread t loads two elements of x row t / 16 and eight of weight row t / 4 per step, and owns the results
 // (row t / 16, columns t % 16 + 16 j).  `x_row` / `w_row` are the thread's rows to load (null: zeros).
 template <typename TX, typename TW>
@@ -157,14 +183,8 @@ __global__ __launch_bounds__(256) void expert_product_mfma_kernel(const bf16_t* 
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + r;
     if (m >= rows) continue;
-    TO* dst = out + (size_t)(first + m) * outputs;
 #pragma unroll
-    for (int s = 0; s < NT; ++s)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = col0 + s * 16 + g * 4 + i;
-        if (n < outputs) dst[n] = from_float<TO>(activation_of(activation, acc[s][t][i]));
-      }
+    for (int s = 0; s < NT; ++s) store_four<TO>(out, (size_t)(first + m), col0 + s * 16 + g * 4, outputs, activation, acc[s][t]);
   }
 }
 
@@ -244,14 +264,8 @@ __global__ __launch_bounds__(256) void expert_tiled_kernel(const bf16_t* __restr
   for (int u = 0; u < 4; ++u) {
     const int m = wave_row + u * 16 + r;
     if (m >= rows) continue;
-    TO* dst = out + (size_t)(first + m) * outputs;
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = col0 + wave_col + s * 16 + g * 4 + i;
-        if (n < outputs) dst[n] = from_float<TO>(activation_of(activation, acc[s][u][i]));
-      }
+    for (int s = 0; s < 4; ++s) store_four<TO>(out, (size_t)(first + m), col0 + wave_col + s * 16 + g * 4, outputs, activation, acc[s][u]);
   }
 }
 
@@ -290,12 +304,7 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(const bf16_t* __rest
   f32x4 total = partial[0][lane];
 #pragma unroll
   for (int v = 1; v < 4; ++v) total += partial[v][lane];
-  TO* dst = out + (size_t)(first + r) * outputs;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int column = blockIdx.x * 16 + g * 4 + i;
-    if (column < outputs) dst[column] = from_float<TO>(activation_of(activation, total[i]));
-  }
+  store_four<TO>(out, (size_t)(first + r), blockIdx.x * 16 + g * 4, outputs, activation, total);
 }
 
 // ---------------------------------------------------------------------------- a product per head
@@ -554,11 +563,19 @@ __global__ __launch_bounds__(256) void expert_product_kernel(const TX* __restric
 // x, w and the first product's result are of one type (bfloat16 or float32); the second product's result is float32.
 // `tile_rows` is what the tiles were made for: 16; or, bfloat16 on the matrix cores only, 64 (K in steps of 32) or 128 (K in
 // steps of 64: operands through LDS).
+// Whether the product of these operands runs on a kernel that can gate its result (ACT_GATED).
+extern "C" int llmserve_expert_product_gates(int is_float, int inner, int tile_rows) {
+  if (is_float) return 0;
+  return tile_rows == TILED_ROWS ? inner % TILED_K == 0 : inner % 32 == 0;
+}
+
 extern "C" int llmserve_expert_product(const void* x, int is_float, const int* order, int top, const void* w, int outputs,
                                        int inner, const int* tiles, int capacity, int tile_rows, void* out, int out_is_float,
                                        int activation, hipStream_t stream) {
   if (capacity <= 0) return 0;
   if (capacity > 65535 || outputs < 1 || inner < 1) return ERR_BAD_ARGUMENT;
+  // a gated result comes from the matrix-core kernels alone, of an even number of columns
+  if (activation >= ACT_GATED && (outputs % 2 || !llmserve_expert_product_gates(is_float, inner, tile_rows))) return ERR_BAD_ARGUMENT;
   if (!is_float && tile_rows == TILED_ROWS) {
     if (inner % TILED_K) return ERR_BAD_ARGUMENT;
     const dim3 through_lds((outputs + TILED_ROWS - 1) / TILED_ROWS, capacity);

@@ -97,9 +97,21 @@ __global__ __launch_bounds__(1024) void stream_norm_kernel(float* __restrict__ s
       squares += u.v[j] * u.v[j];
     }
   }
+  // every thread goes on with the columns it summed itself; the weights of its first piece are asked for before the
+  // workgroup's sum, so that they arrive while it waits
+  struct alignas(sizeof(TO) * V) Normed { TO v[V]; };
+  const int h0 = threadIdx.x * V;
+  float ahead[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) ahead[j] = h0 < width ? load_as_float(weight, weight_is_float, h0 + j) : 0.f;
   const float scale = rsqrtf(block_sum(squares, shared) / (float)width + eps);
-  for (int h = threadIdx.x; h < width; h += blockDim.x)
-    out[(size_t)blockIdx.x * width + h] = from_float<TO>(summed[h] * scale * load_as_float(weight, weight_is_float, h));
+  for (int h = h0; h < width; h += blockDim.x * V) {
+    Normed normed;
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      normed.v[j] = from_float<TO>(summed[h + j] * scale * (h == h0 ? ahead[j] : load_as_float(weight, weight_is_float, h + j)));
+    *(Normed*)(out + (size_t)blockIdx.x * width + h) = normed;
+  }
 }
 
 extern "C" int llmserve_stream_norm(float* streams, const float* result, int parts, int tokens, const float* mix, const float* write,

@@ -21,6 +21,7 @@ from .build import _say, load_module
 _PAIRINGS = {"none": 0, "adjacent": 1, "half": 2}
 # gate activations of a gated product (csrc/elementwise.hip: gate_activation); the products' fused epilogues know silu alone
 _ACTIVATIONS = {"silu": 0, "gelu": 1, "gelu_tanh": 2, "relu": 3}
+_GATED_RESULT = 16  # added to an activation's code: the experts' product gates its own result
 
 
 class KernelError(RuntimeError):
@@ -83,6 +84,7 @@ _SIGNATURES = {
     "llmserve_route": "piipifppiiiiip",
     "llmserve_sort_pairs": "piipppiip",
     "llmserve_expert_product": "pipipiipiipiip",
+    "llmserve_expert_product_gates": "iii",
     "llmserve_combine_pairs": "pppipiippiip",
     "llmserve_conv_gated_delta_rule": "piiipipppppiiiippiiippppppip",
     "llmserve_causal_conv": "piiiipipppipppip",
@@ -1231,15 +1233,20 @@ class HipKernels:
         order = self._empty((pairs,), torch.int32)
         tiles = self._empty((capacity, 3), torch.int32)
         _check(library.llmserve_sort_pairs(_pointer(chosen), pairs, count, _pointer(place), _pointer(order), _pointer(tiles), capacity, tile_rows, self._stream), "experts: sort")
-        inner = self._empty((pairs, size), x.dtype)
+        # the matrix-core kernels gate their result themselves (act(gate) * up of neighbouring columns); behind the others a
+        # kernel of its own does
+        fused = gated and bool(library.llmserve_expert_product_gates(_is_float(x), hidden, tile_rows))
+        code = _ACTIVATIONS[activation] + _GATED_RESULT if fused else -1 if gated else _ACTIVATIONS[activation]
+        inner = self._empty((pairs, width if fused else size), x.dtype)
         _check(library.llmserve_expert_product(
             _pointer(x), _is_float(x), _pointer(order), top, _pointer(ups), size, hidden, _pointer(tiles), capacity, tile_rows, _pointer(inner),
-            _is_float(inner), -1 if gated else _ACTIVATIONS[activation], self._stream), "experts: first product")
-        if gated:  # act(gate) * up of the neighbouring columns
-            both, size = inner, size // 2
-            inner = self._empty((pairs, size), x.dtype)
+            _is_float(inner), code, self._stream), "experts: first product")
+        if gated and not fused:
+            both = inner
+            inner = self._empty((pairs, width), x.dtype)
             _check(self._elementwise.llmserve_gate_mul(
-                _pointer(both), _is_float(both), _pointer(inner), _is_float(inner), pairs, size, _ACTIVATIONS[activation], self._stream), "experts: gate")
+                _pointer(both), _is_float(both), _pointer(inner), _is_float(inner), pairs, width, _ACTIVATIONS[activation], self._stream), "experts: gate")
+        size = width
         rows = self._empty((pairs, hidden), torch.float32)
         _check(library.llmserve_expert_product(
             _pointer(inner), _is_float(inner), _pointer(order), 0, _pointer(downs), hidden, size, _pointer(tiles), capacity, tile_rows, _pointer(rows),
