@@ -38,7 +38,7 @@ def folders(tmp_path_factory):
     wide = cases.config_of(
         [
             (cases.delta(heads=4, kv_heads=2, dim=64, vdim=128, conv=4, decay_rank=16, gate_rank=24), cases.moe(8, 2, 1.5, 64, 128, (4, 2))),
-            (cases.parallel(cases.attention(8, 2, 128, 64, 0.09, 64, base=10000.0, factor=8.0), cases.recurrence(320, 5, 4), 1.1, 0.6),
+            (cases.parallel(cases.attention(8, 2, 128, 64, 0.09, 64, base=10000.0, factor=8.0), cases.recurrence(384, 6, 4), 1.1, 0.6),
              cases.moe(16, 4, 2.0, 32, 96, (4, 3))),
             (cases.delta(heads=2, kv_heads=2, dim=128, vdim=64, conv=2, decay_rank=8, gate_rank=8), None),
             (cases.parallel(cases.attention(4, 4, 64, 64, 0.125, 32, factor=None), cases.recurrence(256, 1, 3), 0.7, 1.4), cases.moe(6, 6, 1.0, 96, None, None)),

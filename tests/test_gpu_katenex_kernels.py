@@ -129,7 +129,7 @@ def test_causal_conv_with_a_bias_and_no_activation(kernels, dtype, taps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,dim,vdim,taps", [(6, 2, 64, 32, 4), (2, 2, 16, 96, 1), (4, 1, 80, 32, 3), (3, 3, 130, 70, 2), (4, 4, 32, 64, 4), (6, 3, 24, 40, 2)])
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,taps", [(6, 2, 64, 32, 4), (2, 2, 16, 96, 1), (4, 1, 80, 32, 3), (3, 3, 130, 70, 2), (5, 5, 32, 48, 3), (6, 3, 24, 40, 2)])
 def test_delta_rule_with_a_decay_per_key_channel(kernels, dtype, heads, kv_heads, dim, vdim, taps):
     """The rule alone and behind its convolutions, over steps of many tokens, of one and of two; the channels' steps are
     the first columns of wider rows, as the part hands them over."""
@@ -177,7 +177,7 @@ def test_head_norm_gated_by_float32_rows(kernels, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,dim,vdim,width,rot", [(6, 2, 24, 40, 48, 10), (3, 1, 16, 16, 16, 16), (8, 4, 96, 96, 96, 48), (2, 1, 70, 6, 80, 6)])
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,width,rot", [(6, 2, 24, 40, 48, 10), (3, 1, 16, 16, 16, 16), (6, 3, 96, 80, 96, 32), (2, 1, 70, 6, 80, 6)])
 def test_heads_turned_in_half_pairs(kernels, dtype, heads, kv_heads, dim, vdim, width, rot):
     torch.manual_seed(heads * dim)
     tokens, extra = 7, 5
@@ -194,8 +194,8 @@ def test_heads_turned_in_half_pairs(kernels, dtype, heads, kv_heads, dim, vdim, 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tokens,experts,top,groups,keep,hidden,size", [
-    (1, 4, 4, 1, 1, 32, 16), (37, 8, 2, 4, 2, 96, 40), (200, 6, 3, 3, 2, 64, 72), (5, 12, 4, 4, 3, 64, 32), (300, 4, 2, 2, 2, 64, 96),
-    (130, 9, 1, 3, 1, 320, 64), (700, 12, 4, 4, 3, 192, 64), (1000, 2, 1, 2, 1, 128, 64), (50, 70, 5, 7, 3, 48, 24),
+    (1, 4, 4, 1, 1, 32, 16), (37, 8, 2, 4, 2, 96, 40), (200, 6, 3, 3, 2, 64, 72), (5, 10, 3, 5, 2, 64, 32), (300, 4, 2, 2, 2, 64, 96),
+    (130, 9, 1, 3, 1, 320, 64), (700, 15, 5, 5, 3, 256, 64), (1000, 2, 1, 2, 1, 128, 64), (50, 70, 5, 7, 3, 48, 24),
 ])
 def test_experts_chosen_within_groups_and_gated(kernels, dtype, tokens, experts, top, groups, keep, hidden, size):
     torch.manual_seed(tokens + experts)
