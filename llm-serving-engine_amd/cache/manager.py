@@ -50,7 +50,8 @@ class SequenceRecord:
     request_id: str
     slot: int
     length: int = 0
-    # per group: number of leading logical blocks already given back (window passed)
+    # per group: the logical blocks below this index have been given back (window passed), except the group's
+    # first `kept` blocks, which hold entries that are read for ever
     released: list[int] = field(default_factory=list)
     last_access_tick: int = 0
 
@@ -177,10 +178,15 @@ class CacheManager:
         return slot
 
     def _first_needed_block(self, group: PageGroup, start: int) -> int:
-        """Blocks below this index hold no key that a query at position >= start reads."""
+        """Blocks below this index (and not among the group's kept ones) hold no key that a query at position >= start reads."""
         if group.need.window is None:
             return 0
         return max(0, start - group.need.window + 1) // self.page_size
+
+    def _kept_blocks(self, group: PageGroup) -> int:
+        """The group's first so many blocks hold entries that every later query reads: a window never gives them back."""
+        keep = int(getattr(group.need, "keep_first", 0) or 0)
+        return -(-keep // self.page_size)
 
     def pages_needed(self, request_id: str, count: int) -> list[tuple[int, int]]:
         """Per group: (pages to allocate, pages given back first) for the next `count` tokens."""
@@ -190,7 +196,7 @@ class CacheManager:
             held_until = math.ceil(record.length / self.page_size)
             wanted_until = math.ceil((record.length + count) / self.page_size)
             first = self._first_needed_block(group, record.length)
-            giving_back = max(0, min(first, held_until) - record.released[index])
+            giving_back = max(0, min(first, held_until) - max(record.released[index], self._kept_blocks(group)))
             need.append((wanted_until - held_until, giving_back))
         return need
 
@@ -241,7 +247,7 @@ class CacheManager:
             table = group.tables[record.slot]
             if group.need.window is not None:
                 first = min(self._first_needed_block(group, start), first_new)
-                for block in range(record.released[index], first):
+                for block in range(max(record.released[index], self._kept_blocks(group)), first):
                     group.pool.free(int(table[block]), request_id)
                     table[block] = -1
                 if first > record.released[index]:
@@ -306,7 +312,9 @@ class CacheManager:
         record = self.sequences[request_id]
         table = group.tables[record.slot]
         page_size = self.page_size
-        for block in range(record.released[group_index], math.ceil(record.length / page_size)):
+        for block in range(math.ceil(record.length / page_size)):
+            if self._kept_blocks(group) <= block < record.released[group_index]:
+                continue  # given back
             held = min(page_size, record.length - block * page_size)
             page = {field: tensor[cell, int(table[block])] for field, tensor in group.storage.items()}
             rows = group.need.token_rows(page, page_size)
@@ -411,7 +419,7 @@ class CacheManager:
                 blocks = math.ceil(record.length / self.page_size)
                 for block in range(self.max_blocks_per_sequence):
                     page = int(table[block])
-                    live = record.released[index] <= block < blocks
+                    live = block < blocks and not self._kept_blocks(group) <= block < record.released[index]
                     if live != (page >= 0):
                         raise AssertionError(f"group {index}: {record.request_id} block {block} holds {page}")
                     if page >= 0:
@@ -442,7 +450,8 @@ class CacheManager:
         held_tokens = 0
         for index, group in enumerate(self.groups):
             for record in self.sequences.values():
-                held_tokens += record.length - record.released[index] * self.page_size
+                given_back = max(0, record.released[index] - self._kept_blocks(group))
+                held_tokens += record.length - given_back * self.page_size
         allocated_slots = used * self.page_size
         waste = allocated_slots - held_tokens
         allocated_bytes = sum(group.pool.used_pages * group.bytes_per_page for group in self.groups)

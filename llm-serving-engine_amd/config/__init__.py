@@ -1,6 +1,8 @@
 from .model import ArchitectureConfig, ConfigError, KeyReader, Qwen2Config
 from .dafutar import DafutarConfig
 from .katenex import KatenexConfig
+from .sozavik import SozavikConfig
+from .vagozen import VagozenConfig
 from .serving import CacheConfig, SchedulerConfig
 
 __all__ = [
@@ -12,4 +14,6 @@ __all__ = [
     "KeyReader",
     "Qwen2Config",
     "SchedulerConfig",
+    "SozavikConfig",
+    "VagozenConfig",
 ]

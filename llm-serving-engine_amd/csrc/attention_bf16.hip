@@ -99,6 +99,7 @@ struct ScoreChange {          // unused unless CHANGED
   const float* slopes;        // [heads], or null
   float soft_cap;             // 0: none
   const float* sinks;         // [heads], or null: exp(sink) more in a head's denominator, once, with no value to it
+  int keep_first;             // under a window, a sequence's first so many keys stay visible to every later query; 0: none
 };
 
 // One step's operands as a lane holds them: its slices of the K rows of the two 16-row tiles and,
@@ -173,7 +174,7 @@ __device__ __forceinline__ void scores_of(const Columns<COLUMN_TILES>& columns, 
 template <int COLUMN_TILES, bool CHANGED = false>
 __device__ __forceinline__ void weigh_and_add(Columns<COLUMN_TILES>& columns, StepLoads& L, const f32x4* s_lo,
                                               const f32x4* s_hi, int key0, int q, bool interior, int last_key,
-                                              int v_start, float scale_log2, float soft_cap = 0.f) {
+                                              int v_start, float scale_log2, float soft_cap = 0.f, int keep = 0) {
   bf16x8 weights[COLUMN_TILES];
 #pragma unroll
   for (int t = 0; t < COLUMN_TILES; ++t) {
@@ -199,9 +200,16 @@ __device__ __forceinline__ void weigh_and_add(Columns<COLUMN_TILES>& columns, St
     if (!interior) {
       // key0 + 8q + i outside [first, position], counted from the lane's first key (nothing to add per key)
       const int last_seen = columns.position[t] - (key0 + 8 * q), first_seen = columns.first[t] - (key0 + 8 * q);
+      if constexpr (CHANGED) {  // (the sequence's first `keep` keys are seen whatever the window)
+        const int kept_seen = keep - (key0 + 8 * q);
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (i > last_seen || i < first_seen) x[i] = -INFINITY;
+        for (int i = 0; i < 8; ++i)
+          if (i > last_seen || (i < first_seen && i >= kept_seen)) x[i] = -INFINITY;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (i > last_seen || i < first_seen) x[i] = -INFINITY;
+      }
     }
     // (the largest of three in one instruction, written out: through fmaxf the compiler first passes every
     // score through a v_max with itself, thirteen instructions for eight scores where four do)
@@ -391,8 +399,16 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
   }
 
   const int step_first = first_key / KEYS, step_last = last_key / KEYS;
-  const int per_split = (step_last - step_first + 1 + splits - 1) / splits;
-  const int step_begin = step_first + blockIdx.z * per_split;
+  // CHANGED with `keep_first`: the sequence's first `keep` keys stay visible behind a window.  Those of them that lie in
+  // steps before the window's first are walked first: the walk counts from step_first - kept_steps, and a step below
+  // step_first stands for step (it - step_first + kept_steps) of the sequence's start.  (Kept keys within the window's
+  // first step are read there.)  Without kept keys the walk is the window's, as it was.
+  const int keep = CHANGED ? change.keep_first : 0;
+  const int kept_steps = CHANGED ? min((min(keep, first_key) + KEYS - 1) / KEYS, step_first) : 0;
+  const int walk_first = step_first - kept_steps;
+  auto real_step = [&](int step) { return CHANGED && step < step_first ? step - walk_first : step; };
+  const int per_split = (step_last - walk_first + 1 + splits - 1) / splits;
+  const int step_begin = walk_first + blockIdx.z * per_split;
   const int step_end = min(step_last + 1, step_begin + per_split);
   const unsigned page_stride = (unsigned)kv_heads * page_size * D;  // elements of one page: checked to fit by the host
   const unsigned head_offset = (unsigned)kv_head * page_size * D;
@@ -446,13 +462,31 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
   // within the pages are arithmetic.
   struct StepPages { int k, k_hi, v; };
   struct StepKeys { int k, k_hi, v; };
+  // (a kept key is read where it lies; a key between the kept ones and the window's first counts as outside, and a
+  // piece of eight values that begins with a kept key lies in a page that is kept)
+  auto held_key = [&](int key) {
+    if constexpr (CHANGED) {
+      key = min(key, last_key);
+      return key < first_key && key >= keep ? first_key : key;
+    } else {
+      return min(max(key, first_key), last_key);
+    }
+  };
+  auto held_piece = [&](int key) {
+    if constexpr (CHANGED) {
+      key = min(key, high_limit);
+      return key < low_limit && key >= keep ? low_limit : key;
+    } else {
+      return min(max(key, low_limit), high_limit);
+    }
+  };
   auto keys_of = [&](int step) {  // the keys this lane reads in a step
-    const int key0 = step * KEYS;
+    const int key0 = real_step(step) * KEYS;
     StepKeys at = {key0 + row_key, key0 + row_key + 4, key0 + 8 * q};
     if (key0 < first_key || key0 + KEYS - 1 > last_key) {
-      at.k = min(max(at.k, first_key), last_key);
-      at.k_hi = min(max(at.k_hi, first_key), last_key);
-      at.v = min(max(at.v, low_limit), high_limit);
+      at.k = held_key(at.k);
+      at.k_hi = held_key(at.k_hi);
+      at.v = held_piece(at.v);
     }
     return at;
   };
@@ -539,10 +573,10 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
       f32x4 s_lo[COLUMN_TILES], s_hi[COLUMN_TILES];
       scores_of(columns, loads, s_lo, s_hi);
       if (more) fetch_keys(step + WAVES, pages, loads);
-      const int key0 = step * KEYS;
+      const int key0 = real_step(step) * KEYS;
       const bool interior = key0 + KEYS - 1 <= position0 && (window <= 0 || key0 >= last_key - window + 1);
-      weigh_and_add<COLUMN_TILES, CHANGED>(columns, loads, s_lo, s_hi, key0, q, interior, last_key,
-                                           min(max(key0 + 8 * q, low_limit), high_limit), scale_log2, change.soft_cap);
+      weigh_and_add<COLUMN_TILES, CHANGED>(columns, loads, s_lo, s_hi, key0, q, interior, last_key, held_piece(key0 + 8 * q),
+                                           scale_log2, change.soft_cap, keep);
       if (more) fetch_values(step + WAVES, pages, loads);
       if (step + 2 * WAVES < step_end) pages = pages_of(step + 2 * WAVES);
     }
@@ -1000,7 +1034,7 @@ static int launch_tiles(const void* qkv, int row_width, void* out, float* partia
                         void* keys, void* values, const int* block_tables, int table_width,
                         const int* positions, const int* work, int tiles, int heads, int kv_heads,
                         int tokens_per_tile, int page_size, float scale, int window, int splits, FusedDecode fused,
-                        hipStream_t stream, ScoreChange change = {nullptr, 0.f, nullptr}) {
+                        hipStream_t stream, ScoreChange change = {nullptr, 0.f, nullptr, 0}) {
   const int group = heads / kv_heads;
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
   const int head_tiles = (group + 15) / 16;
@@ -1047,18 +1081,21 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 // weights, and partial_ml [heads][splits][16 rows][2] holds each split's maximum (in units of log2) and sum of
 // weights.
 // `slopes` (float32 [heads], or null) and `soft_cap` (0 for none) change the scores before the softmax (see the head of
-// this file), `sinks` (float32 [heads], or null) add exp(sink) to a head's denominator; not together with `fuse` & 1.
+// this file), `sinks` (float32 [heads], or null) add exp(sink) to a head's denominator, `keep_first` keeps a sequence's first
+// keys visible behind a window; not together with `fuse` & 1.
 extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* out, float* partial_acc,
                                         float* partial_ml, void* keys, void* values,
                                         const int* block_tables, int table_width, const int* positions,
                                         const int* work, int tiles, int column_tiles, int rows, int heads,
                                         int kv_heads, int page_size, float scale, int window, int splits, int fuse,
                                         const float* table, int pairing, const int* slots, const float* slopes,
-                                        float soft_cap, const float* sinks, hipStream_t stream) {
+                                        float soft_cap, const float* sinks, int keep_first, hipStream_t stream) {
   if (tiles <= 0) return 0;
-  const bool changed = slopes != nullptr || soft_cap > 0.f || sinks != nullptr;
+  if (keep_first < 0) return ERR_BAD_ARGUMENT;
+  if (window <= 0) keep_first = 0;  // (without a window every key is seen anyway)
+  const bool changed = slopes != nullptr || soft_cap > 0.f || sinks != nullptr || keep_first > 0;
   if (soft_cap < 0.f || (changed && (fuse & 1)) || (sinks && (fuse & 2))) return ERR_BAD_ARGUMENT;
-  const ScoreChange change = {slopes, soft_cap, sinks};
+  const ScoreChange change = {slopes, soft_cap, sinks, keep_first};
   if (heads % kv_heads || page_size % 8 || splits < 1 || splits > MERGE_SPLITS_MAX || (splits > 1 && (!partial_acc || !partial_ml)))
     return ERR_BAD_ARGUMENT;
   if ((long)kv_heads * page_size * D >= (1L << 31)) return ERR_BAD_ARGUMENT;  // a page's elements are counted in 32 bits

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
     float* __restrict__ partial_ml, const float* __restrict__ keys, const float* __restrict__ values,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ positions,
     const int* __restrict__ work, int heads, int kv_heads, int page_size, float scale_log2, int window, int splits,
-    int columns_total, const float* __restrict__ slopes, float soft_cap, const float* __restrict__ sinks) {
+    int columns_total, const float* __restrict__ slopes, float soft_cap, const float* __restrict__ sinks, int keep_first) {
   __shared__ float wave_max[WAVES][COLUMN_TILES][16];
   __shared__ float wave_sum[WAVES][COLUMN_TILES][16];
   __shared__ __attribute__((aligned(16))) float merged[COLUMN_TILES][D_STEPS][64][4];
@@ -90,8 +90,15 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
   const int begin = window > 0 ? max(0, first_position - window + 1) : 0;
   // steps of 16 keys, aligned to 16; the splits share them in contiguous runs, the waves take a run's in turn
   const int step_first = begin / KEYS, step_end = (end + KEYS - 1) / KEYS;
-  const int per_split = (step_end - step_first + splits - 1) / splits;
-  const int my_first = step_first + split * per_split, my_end = min(step_end, my_first + per_split);
+  // The sequence's first `keep` keys stay visible behind a window.  Those of them that lie in steps before the window's
+  // first are walked first: the walk counts from step_first - kept_steps, and a step below step_first stands for step
+  // (it - step_first + kept_steps) of the sequence's start.  (Kept keys within the window's first step are read there.)
+  const int keep = CHANGED ? keep_first : 0;
+  const int kept_steps = min((min(keep, begin) + KEYS - 1) / KEYS, step_first);
+  const int walk_first = step_first - kept_steps;
+  const int per_split = (step_end - walk_first + splits - 1) / splits;
+  const int my_first = walk_first + split * per_split, my_end = min(step_end, my_first + per_split);
+  auto real_step = [&](int step) { return step < step_first ? step - walk_first : step; };
 
   float running_max[COLUMN_TILES], running_sum[COLUMN_TILES];
   f32x4 acc[COLUMN_TILES][D_STEPS];
@@ -108,15 +115,22 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
   // Which key a lane reads for the first product (key0 + i) and which four for the second (key0 + 4 g .. + 3, one
   // page: pages are multiples of 4).  A key outside the item's range is masked, and its page may have been given
   // back: the nearest inside is read instead.  The pages of a wave's next step are looked up a step ahead.
-  auto key_of = [&](int step) { return max(min(step * KEYS + i, end - 1), begin); };
-  auto value_key_of = [&](int step) { return max(min(step * KEYS + 4 * g, (end - 1) & ~3), begin & ~3); };
+  // (a kept key is read where it lies; a key between the kept ones and the window's first counts as outside)
+  auto key_of = [&](int step) {
+    const int key = min(real_step(step) * KEYS + i, end - 1);
+    return key < begin && key >= keep ? begin : key;
+  };
+  auto value_key_of = [&](int step) {
+    const int key = min(real_step(step) * KEYS + 4 * g, (end - 1) & ~3);
+    return key < (begin & ~3) && key >= keep ? begin & ~3 : key;
+  };
   int next_key_page = 0, next_value_page = 0;
   if (my_first + wave < my_end) {
     next_key_page = table[key_of(my_first + wave) / page_size];
     next_value_page = table[value_key_of(my_first + wave) / page_size];
   }
   for (int step = my_first + wave; step < my_end; step += WAVES) {
-    const int key0 = step * KEYS;
+    const int key0 = real_step(step) * KEYS;
     // K: lane (i, g) reads d = 16 s + 4 g .. + 3 of its key
     const int key_mine = key_of(step);
     const int key_page = next_key_page;
@@ -153,7 +167,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int key = key0 + 4 * g + e;
-        const bool seen = key <= position[t] && key >= first[t];
+        const bool seen = key <= position[t] && (key >= first[t] || key < keep);
         if (CHANGED) {  // scores are kept in units of log2: the cap is applied to the score itself
           if (soft_cap > 0.f) s4[e] = soft_cap * 1.4426950408889634f * tanhf(s4[e] * 0.6931471805599453f / soft_cap);
           s4[e] -= slope[t] * (float)(position[t] - key);
@@ -323,19 +337,20 @@ extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* ou
                                       const float* keys, const float* values, const int* block_tables, int table_width,
                                       const int* positions, const int* work, int items, int column_tiles, int tokens,
                                       int heads, int kv_heads, int page_size, float scale, int window, int splits,
-                                      const float* slopes, float soft_cap, const float* sinks, hipStream_t stream) {
+                                      const float* slopes, float soft_cap, const float* sinks, int keep_first, hipStream_t stream) {
   if (items <= 0 || tokens <= 0) return 0;
+  if (keep_first < 0) return ERR_BAD_ARGUMENT;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 4 || splits < 1 ||
       splits > MERGE_SPLITS_MAX || (column_tiles != 1 && column_tiles != 2) || (splits > 1 && (!partial_acc || !partial_ml)))
     return ERR_BAD_ARGUMENT;
   const float scale_log2 = scale * 1.4426950408889634f;
   const int columns_total = tokens * heads;
   dim3 grid(items, kv_heads, splits);
-  const bool changed = slopes != nullptr || soft_cap > 0.f || sinks != nullptr;
+  const bool changed = slopes != nullptr || soft_cap > 0.f || sinks != nullptr || (keep_first > 0 && window > 0);
 #define LAUNCH_ATTENTION_F32(TILES, CHANGED)                                                                          \
   hipLaunchKernelGGL((attention_f32_kernel<TILES, CHANGED>), grid, dim3(WAVES * 64), 0, stream, qkv, row_width, out,   \
                      partial_acc, partial_ml, keys, values, block_tables, table_width, positions, work, heads,        \
-                     kv_heads, page_size, scale_log2, window, splits, columns_total, slopes, soft_cap, sinks)
+                     kv_heads, page_size, scale_log2, window, splits, columns_total, slopes, soft_cap, sinks, keep_first)
   if (column_tiles == 1 && !changed) LAUNCH_ATTENTION_F32(1, false);
   else if (column_tiles == 1) LAUNCH_ATTENTION_F32(1, true);
   else if (!changed) LAUNCH_ATTENTION_F32(2, false);

@@ -20,7 +20,8 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
     const T* __restrict__ qkv, int row_width, T* __restrict__ out, const T* __restrict__ keys,
     const T* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ token_sequence, const int* __restrict__ positions, int heads, int kv_heads, int dim,
-    int page_size, float scale, int window, const float* __restrict__ slopes, float soft_cap, const float* __restrict__ sinks) {
+    int page_size, float scale, int window, const float* __restrict__ slopes, float soft_cap, const float* __restrict__ sinks,
+    int keep_first) {
   __shared__ float query[MAX_DIM];
   __shared__ float weights[KEYS_PER_TILE];
   __shared__ float shared[17];
@@ -39,8 +40,12 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
   float acc[MAX_DIM / KEYS_PER_TILE] = {};
   float running_max = -INFINITY, running_sum = 0.f;
 
-  for (int tile = first; tile <= position; tile += KEYS_PER_TILE) {
-    const int key = tile + threadIdx.x;
+  // The keys a query sees, counted through: the sequence's first `kept` keys (those of its first `keep_first` that the
+  // window has passed; they stay visible at their own positions), then the window's.
+  const int kept = min(keep_first, first), seen = kept + position - first + 1;
+  auto key_of = [&](int index) { return index < kept ? index : first + index - kept; };
+  for (int tile = 0; tile < seen; tile += KEYS_PER_TILE) {
+    const int key = key_of(tile + threadIdx.x);
     float score = -INFINITY;
     if (key <= position) {
       const int page = table[key / page_size];
@@ -63,13 +68,13 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
     const float tile_sum = block_sum(weight, shared);  // also orders the writes to `weights`
     running_sum = running_sum * correction + tile_sum;
     running_max = next_max;
-    const int in_tile = min(KEYS_PER_TILE, position - tile + 1);
+    const int in_tile = min(KEYS_PER_TILE, seen - tile);
     for (int i = 0; i < per_thread; ++i) {
       const int d = threadIdx.x + i * KEYS_PER_TILE;
       if (d >= dim) break;
       float sum = 0.f;
       for (int j = 0; j < in_tile; ++j) {
-        const int at = tile + j;
+        const int at = key_of(tile + j);
         const int page = table[at / page_size];
         const T* v = values + ((size_t)page * kv_heads + kv_head) * page_size * dim;
         sum = fmaf(weights[j], to_float(v[value_element(d, at % page_size, page_size, dim)]), sum);  // common.h: value_element
@@ -95,17 +100,18 @@ extern "C" int llmserve_attention_generic(const void* qkv, int row_width, void* 
                                           const void* values, const int* block_tables, int table_width,
                                           const int* token_sequence, const int* positions, int tokens, int heads,
                                           int kv_heads, int dim, int page_size, float scale, int window,
-                                          const float* slopes, float soft_cap, const float* sinks, hipStream_t stream) {
+                                          const float* slopes, float soft_cap, const float* sinks, int keep_first,
+                                          hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (dim > MAX_DIM || dim <= 0 || heads % kv_heads || page_size <= 0) return ERR_BAD_ARGUMENT;
+  if (dim > MAX_DIM || dim <= 0 || heads % kv_heads || page_size <= 0 || keep_first < 0) return ERR_BAD_ARGUMENT;
   dim3 grid(tokens, heads);
   if (is_float)
     hipLaunchKernelGGL(attention_generic_kernel<float>, grid, dim3(KEYS_PER_TILE), 0, stream, (const float*)qkv,
                        row_width, (float*)out, (const float*)keys, (const float*)values, block_tables, table_width,
-                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap, sinks);
+                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap, sinks, keep_first);
   else
     hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, dim3(KEYS_PER_TILE), 0, stream, (const bf16_t*)qkv,
                        row_width, (bf16_t*)out, (const bf16_t*)keys, (const bf16_t*)values, block_tables, table_width,
-                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap, sinks);
+                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap, sinks, keep_first);
   return LAUNCH_STATUS();
 }

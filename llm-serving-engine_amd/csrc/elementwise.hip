@@ -546,6 +546,14 @@ extern "C" int llmserve_rotate_and_store(void* qkv, int is_float, const float* t
 #define ACT_GELU 1
 #define ACT_GELU_TANH 2
 #define ACT_RELU 3
+// 4: a function of gate and up both, with a limit: g = min(gate, limit), u = clamp(up, -limit, limit),
+// g * sigmoid(1.702 g) * (u + 1)
+#define ACT_LIMITED_SWISH 4
+
+__device__ __forceinline__ float limited_swish(float gate, float up, float limit) {
+  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+  return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+}
 
 __device__ __forceinline__ float gate_activation(int activation, float z) {
   switch (activation) {
@@ -557,13 +565,30 @@ __device__ __forceinline__ float gate_activation(int activation, float z) {
 }
 
 template <typename TI, typename TO>
-__global__ void gate_mul_kernel(const TI* __restrict__ in, TO* __restrict__ out, int width, int activation) {
+__global__ void gate_mul_kernel(const TI* __restrict__ in, TO* __restrict__ out, int width, int activation, float limit) {
   const TI* row = in + (size_t)blockIdx.x * 2 * width;
   TO* dst = out + (size_t)blockIdx.x * width;
   for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < width; i += gridDim.y * blockDim.x) {
     const float gate = to_float(row[2 * i]), up = to_float(row[2 * i + 1]);
-    dst[i] = from_float<TO>(gate_activation(activation, gate) * up);
+    dst[i] = from_float<TO>(activation == ACT_LIMITED_SWISH ? limited_swish(gate, up, limit) : gate_activation(activation, gate) * up);
   }
+}
+
+// The limited gate for bfloat16 rows whose width is a multiple of 8: a thread takes eight outputs, 32 bytes in (two
+// 16-byte loads, both on their way before the first is used) and 16 bytes out.
+__global__ __launch_bounds__(256) void limited_swish_vector_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out,
+                                                                   size_t octets, float limit) {
+  typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+  const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (at >= octets) return;
+  const bf16x8 first = ((const bf16x8*)in)[2 * at], second = ((const bf16x8*)in)[2 * at + 1];
+  bf16x8 result;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    result[i] = (bf16_t)limited_swish((float)first[2 * i], (float)first[2 * i + 1], limit);
+    result[4 + i] = (bf16_t)limited_swish((float)second[2 * i], (float)second[2 * i + 1], limit);
+  }
+  ((bf16x8*)out)[at] = result;
 }
 
 // SiLU for bfloat16 rows whose width is a multiple of 8: a thread takes eight outputs, 32 bytes in
@@ -585,10 +610,16 @@ __global__ __launch_bounds__(256) void silu_mul_vector_kernel(const bf16_t* __re
   ((bf16x8*)out)[at] = result;
 }
 
-extern "C" int llmserve_gate_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
-                                 int activation, hipStream_t stream) {
+extern "C" int llmserve_gate_mul_limit(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
+                                       int activation, float limit, hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (activation < ACT_SILU || activation > ACT_RELU) return ERR_BAD_ARGUMENT;
+  if (activation < ACT_SILU || activation > ACT_LIMITED_SWISH || (activation == ACT_LIMITED_SWISH && !(limit > 0.f))) return ERR_BAD_ARGUMENT;
+  if (activation == ACT_LIMITED_SWISH && !in_is_float && !out_is_float && width % 8 == 0) {
+    const size_t octets = (size_t)rows * (width / 8);
+    hipLaunchKernelGGL(limited_swish_vector_kernel, dim3((unsigned)((octets + 255) / 256)), dim3(256), 0, stream,
+                       (const bf16_t*)in, (bf16_t*)out, octets, limit);
+    return LAUNCH_STATUS();
+  }
   if (activation == ACT_SILU && !in_is_float && !out_is_float && width % 8 == 0) {  // rows are contiguous: one run of octets
     const size_t octets = (size_t)rows * (width / 8);
     hipLaunchKernelGGL(silu_mul_vector_kernel, dim3((unsigned)((octets + 255) / 256)), dim3(256), 0, stream,
@@ -599,14 +630,20 @@ extern "C" int llmserve_gate_mul(const void* in, int in_is_float, void* out, int
   const int pieces = rows >= 1024 ? 1 : max(1, min((width + 255) / 256, 1024 / rows));
   const dim3 grid(rows, pieces), block(256);
   if (in_is_float && out_is_float)
-    hipLaunchKernelGGL((gate_mul_kernel<float, float>), grid, block, 0, stream, (const float*)in, (float*)out, width, activation);
+    hipLaunchKernelGGL((gate_mul_kernel<float, float>), grid, block, 0, stream, (const float*)in, (float*)out, width, activation, limit);
   else if (in_is_float)
-    hipLaunchKernelGGL((gate_mul_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)in, (bf16_t*)out, width, activation);
+    hipLaunchKernelGGL((gate_mul_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)in, (bf16_t*)out, width, activation, limit);
   else if (out_is_float)
-    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, float>), grid, block, 0, stream, (const bf16_t*)in, (float*)out, width, activation);
+    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, float>), grid, block, 0, stream, (const bf16_t*)in, (float*)out, width, activation, limit);
   else
-    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, width, activation);
+    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, width, activation, limit);
   return LAUNCH_STATUS();
+}
+
+extern "C" int llmserve_gate_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,
+                                 int activation, hipStream_t stream) {
+  if (activation == ACT_LIMITED_SWISH) return ERR_BAD_ARGUMENT;  // (that one has a limit: llmserve_gate_mul_limit)
+  return llmserve_gate_mul_limit(in, in_is_float, out, out_is_float, rows, width, activation, 0.f, stream);
 }
 
 extern "C" int llmserve_silu_mul(const void* in, int in_is_float, void* out, int out_is_float, int rows, int width,

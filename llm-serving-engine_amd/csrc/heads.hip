@@ -1,6 +1,9 @@
 // Operations around attention heads and around norms that act on a sublayer's result:
 //   stream_rows     hidden += delta; the rows in the run dtype
-//   add_normed      hidden += rms_norm(update) * weight; the rows in the run dtype
+//   add_normed      hidden += rms_norm(update) * weight; the rows in the run dtype, or, with the weight of a next norm,
+//                   rms_norm(hidden) * that weight: the norm behind a sublayer, the add and the norm before the next in one
+//   rotate_heads    a run of heads of a row turned in pairs by the token's angles and scaled, in place
+//   add_rows        hidden += delta (+ other rows) (+ one vector for all rows)
 //   assemble_heads  queries, keys and values of a projected row normed, turned, blended and widened to one head width
 //   scale_heads     every head of a row times the squashed gate of that head
 //   soft_cap        cap * tanh(x / cap)
@@ -74,7 +77,9 @@ __device__ __forceinline__ void add_some_parts(float4 (&v)[PIECES], const float*
 template <typename TO, int PIECES>
 __global__ __launch_bounds__(1024) void add_normed_vector_kernel(float* __restrict__ hidden, const float* __restrict__ update,
                                                                  int parts, size_t part_stride, const void* __restrict__ weight,
-                                                                 int weight_is_float, TO* __restrict__ out, int width, float eps) {
+                                                                 int weight_is_float, TO* __restrict__ out, int width, float eps,
+                                                                 const void* __restrict__ next_weight, int next_is_float,
+                                                                 float next_eps) {
   __shared__ float shared[17];
   const int quads = width / 4;
   float4* row = (float4*)(hidden + (size_t)blockIdx.x * width);
@@ -110,15 +115,43 @@ __global__ __launch_bounds__(1024) void add_normed_vector_kernel(float* __restri
       const float4 r = make_float4(h[j].x + u[j].x * scale * w.x, h[j].y + u[j].y * scale * w.y, h[j].z + u[j].z * scale * w.z,
                                    h[j].w + u[j].w * scale * w.w);
       row[i] = r;
-      if (out) store_four(out + (size_t)blockIdx.x * width + 4 * i, r.x, r.y, r.z, r.w);
+      h[j] = r;
+      if (out && !next_weight) store_four(out + (size_t)blockIdx.x * width + 4 * i, r.x, r.y, r.z, r.w);
     }
+  }
+  if (!next_weight) return;  // (the same for the whole block)
+  // the norm before the next sublayer, of the row as it now is: its weight is asked for ahead of the block's sum
+  float4 next[PIECES];
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = min((int)(threadIdx.x + j * blockDim.x), quads - 1);
+    if (next_is_float) {
+      next[j] = ((const float4*)next_weight)[i];
+    } else {
+      const uint2 raw = ((const uint2*)next_weight)[i];
+      next[j] = make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                            __uint_as_float(raw.y & 0xffff0000u));
+    }
+  }
+  float again = 0.f;
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j)
+    if ((int)(threadIdx.x + j * blockDim.x) < quads) again += h[j].x * h[j].x + h[j].y * h[j].y + h[j].z * h[j].z + h[j].w * h[j].w;
+  const float next_scale = rsqrtf(block_sum(again, shared) / (float)width + next_eps);
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    if (i < quads)
+      store_four(out + (size_t)blockIdx.x * width + 4 * i, h[j].x * next_scale * next[j].x, h[j].y * next_scale * next[j].y,
+                 h[j].z * next_scale * next[j].z, h[j].w * next_scale * next[j].w);
   }
 }
 
 template <typename TO>
 __global__ __launch_bounds__(256) void add_normed_kernel(float* __restrict__ hidden, const float* __restrict__ update, int parts,
                                                          size_t part_stride, const void* __restrict__ weight, int weight_is_float,
-                                                         TO* __restrict__ out, int width, float eps) {
+                                                         TO* __restrict__ out, int width, float eps,
+                                                         const void* __restrict__ next_weight, int next_is_float, float next_eps) {
   __shared__ float shared[17];
   float* row = hidden + (size_t)blockIdx.x * width;
   const float* from = update + (size_t)blockIdx.x * width;
@@ -134,13 +167,20 @@ __global__ __launch_bounds__(256) void add_normed_kernel(float* __restrict__ hid
     for (int p = 1; p < parts; ++p) u += from[p * part_stride + i];
     const float r = row[i] + u * scale * load_as_float(weight, weight_is_float, i);
     row[i] = r;
-    if (out) out[(size_t)blockIdx.x * width + i] = from_float<TO>(r);
+    if (out && !next_weight) out[(size_t)blockIdx.x * width + i] = from_float<TO>(r);
   }
+  if (!next_weight) return;
+  float again = 0.f;  // (a thread reads back what it wrote itself)
+  for (int i = threadIdx.x; i < width; i += blockDim.x) again += row[i] * row[i];
+  const float next_scale = rsqrtf(block_sum(again, shared) / (float)width + next_eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    out[(size_t)blockIdx.x * width + i] = from_float<TO>(row[i] * next_scale * load_as_float(next_weight, next_is_float, i));
 }
 
 template <typename TO>
 static void launch_add_normed(float* hidden, const float* update, int parts, const void* weight, int weight_is_float, TO* out,
-                              int rows, int width, float eps, hipStream_t stream) {
+                              int rows, int width, float eps, hipStream_t stream, const void* next_weight = nullptr,
+                              int next_is_float = 0, float next_eps = 0.f) {
   const size_t part_stride = (size_t)rows * width;
   if (width % 4 == 0 && width <= 1024 * 4 * 4) {
     const int quads = width / 4;
@@ -148,17 +188,17 @@ static void launch_add_normed(float* hidden, const float* update, int parts, con
     const int threads = ((quads + pieces - 1) / pieces + WAVE - 1) / WAVE * WAVE;
     if (pieces == 1)
       hipLaunchKernelGGL((add_normed_vector_kernel<TO, 1>), dim3(rows), dim3(threads), 0, stream, hidden, update, parts, part_stride,
-                         weight, weight_is_float, out, width, eps);
+                         weight, weight_is_float, out, width, eps, next_weight, next_is_float, next_eps);
     else if (pieces == 2)
       hipLaunchKernelGGL((add_normed_vector_kernel<TO, 2>), dim3(rows), dim3(threads), 0, stream, hidden, update, parts, part_stride,
-                         weight, weight_is_float, out, width, eps);
+                         weight, weight_is_float, out, width, eps, next_weight, next_is_float, next_eps);
     else
       hipLaunchKernelGGL((add_normed_vector_kernel<TO, 4>), dim3(rows), dim3(threads), 0, stream, hidden, update, parts, part_stride,
-                         weight, weight_is_float, out, width, eps);
+                         weight, weight_is_float, out, width, eps, next_weight, next_is_float, next_eps);
     return;
   }
   hipLaunchKernelGGL(add_normed_kernel<TO>, dim3(rows), dim3(256), 0, stream, hidden, update, parts, part_stride, weight,
-                     weight_is_float, out, width, eps);
+                     weight_is_float, out, width, eps, next_weight, next_is_float, next_eps);
 }
 
 // `out` null, or bfloat16 rows (out_is_float 0), or float32 rows
@@ -170,6 +210,88 @@ extern "C" int llmserve_add_normed(float* hidden, const float* update, int parts
     launch_add_normed<float>(hidden, update, parts, weight, weight_is_float, (float*)out, rows, width, eps, stream);
   else
     launch_add_normed<bf16_t>(hidden, update, parts, weight, weight_is_float, (bf16_t*)out, rows, width, eps, stream);
+  return LAUNCH_STATUS();
+}
+
+// The same, and then the norm before the next sublayer: out = new row * rsqrt(mean(new row^2) + next_eps) * next_weight.
+extern "C" int llmserve_add_normed_norm(float* hidden, const float* update, int parts, const void* weight, int weight_is_float,
+                                        float eps, const void* next_weight, int next_is_float, float next_eps, void* out,
+                                        int out_is_float, int rows, int width, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (!update || !next_weight || !out || parts < 1 || width < 1) return ERR_BAD_ARGUMENT;
+  if (out_is_float)
+    launch_add_normed<float>(hidden, update, parts, weight, weight_is_float, (float*)out, rows, width, eps, stream, next_weight,
+                             next_is_float, next_eps);
+  else
+    launch_add_normed<bf16_t>(hidden, update, parts, weight, weight_is_float, (bf16_t*)out, rows, width, eps, stream, next_weight,
+                              next_is_float, next_eps);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- heads turned in place
+// For every token and every one of `heads` heads (`head_stride` columns each, from column `first` of a row `x_width`
+// wide): the first `dims` columns turn in pairs (pairing 1: (2i, 2i + 1); 2: (i, i + dims / 2)) by (cos, sin) of
+// table[token][i], and every column of the head is multiplied by `scale`.  float32 arithmetic; a thread a pair, or a
+// column beyond the pairs.
+template <typename T>
+__global__ __launch_bounds__(256) void rotate_heads_kernel(T* __restrict__ x, int x_width, int first, int head_stride, int heads,
+                                                           const float* __restrict__ table, int dims, int pairing, float scale) {
+  const size_t token = blockIdx.x;
+  T* row = x + token * x_width + first;
+  const int half = dims / 2, per_head = head_stride - half;  // work items a head: the pairs, then the columns left
+  for (int item = threadIdx.x; item < heads * per_head; item += blockDim.x) {
+    const int head = item / per_head, inside = item - head * per_head;
+    T* at = row + (size_t)head * head_stride;
+    if (inside < half) {
+      const int a_at = pairing == 1 ? 2 * inside : inside, b_at = pairing == 1 ? 2 * inside + 1 : inside + half;
+      const float2 cs = ((const float2*)table)[token * half + inside];
+      const float a = to_float(at[a_at]), b = to_float(at[b_at]);
+      at[a_at] = from_float<T>((a * cs.x - b * cs.y) * scale);
+      at[b_at] = from_float<T>((b * cs.x + a * cs.y) * scale);
+    } else if (scale != 1.f) {
+      const int column = dims + inside - half;
+      at[column] = from_float<T>(to_float(at[column]) * scale);
+    }
+  }
+}
+
+extern "C" int llmserve_rotate_heads(void* x, int is_float, int tokens, int x_width, int first, int head_stride, int heads,
+                                     const float* table, int dims, int pairing, float scale, hipStream_t stream) {
+  if (tokens <= 0 || heads <= 0) return 0;
+  if (dims < 0 || dims % 2 || dims > head_stride || first < 0 || first + heads * head_stride > x_width || (dims > 0 && !table) ||
+      (dims > 0 && pairing != 1 && pairing != 2))
+    return ERR_BAD_ARGUMENT;
+  if (is_float)
+    hipLaunchKernelGGL(rotate_heads_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float*)x, x_width, first, head_stride, heads,
+                       table, dims, pairing, scale);
+  else
+    hipLaunchKernelGGL(rotate_heads_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t*)x, x_width, first, head_stride, heads,
+                       table, dims, pairing, scale);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- rows and a vector added to the stream
+// hidden[t] += delta[0][t] + delta[1][t] + ... (+ other[t]) (+ vector), float32, in place; any of the three may be null.
+__global__ __launch_bounds__(256) void add_rows_kernel(float* __restrict__ hidden, const float* __restrict__ delta, int parts,
+                                                       size_t part_stride, const float* __restrict__ other,
+                                                       const float* __restrict__ vector, int width, size_t count) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float v = hidden[i];
+  if (delta)
+    for (int p = 0; p < parts; ++p) v += delta[p * part_stride + i];
+  if (other) v += other[i];
+  if (vector) v += vector[i % width];
+  hidden[i] = v;
+}
+
+extern "C" int llmserve_add_rows(float* hidden, const float* delta, int parts, const float* other, const float* vector, int rows,
+                                 int width, hipStream_t stream) {
+  if (rows <= 0 || (!delta && !other && !vector)) return 0;
+  if (delta && parts < 1) return ERR_BAD_ARGUMENT;
+  const size_t count = (size_t)rows * width;
+  hipLaunchKernelGGL(add_rows_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, hidden, delta, parts, count, other,
+                     vector, width, count);
   return LAUNCH_STATUS();
 }
 

@@ -20,7 +20,7 @@ from .build import _say, load_module
 
 _PAIRINGS = {"none": 0, "adjacent": 1, "half": 2}
 # gate activations of a gated product (csrc/elementwise.hip: gate_activation); the products' fused epilogues know silu alone
-_ACTIVATIONS = {"silu": 0, "gelu": 1, "gelu_tanh": 2, "relu": 3}
+_ACTIVATIONS = {"silu": 0, "gelu": 1, "gelu_tanh": 2, "relu": 3, "limited_swish": 4}  # (the last is a function of gate and up both, with a limit)
 _GATED_RESULT = 16  # added to an activation's code: the experts' product gates its own result
 
 
@@ -54,6 +54,10 @@ _SIGNATURES = {
     "llmserve_rotate_and_store": "pipiiiiipppip",
     "llmserve_silu_mul": "pipiiip",
     "llmserve_gate_mul": "pipiiiip",
+    "llmserve_gate_mul_limit": "pipiiiifp",
+    "llmserve_add_normed_norm": "ppipifpifpiiip",
+    "llmserve_rotate_heads": "piiiiiipiifp",
+    "llmserve_add_rows": "ppippiip",
     "llmserve_gather_rows": "ppiippiip",
     "llmserve_gemm_generic": "pipipipiiiip",
     "llmserve_gemm_f32": "ppppiiiiip",
@@ -64,9 +68,9 @@ _SIGNATURES = {
     "llmserve_gemm_ring": "pppipiiiiiiip",
     "llmserve_gemm_merged": "ppippipiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",
-    "llmserve_attention_generic": "pipipppippiiiiifipfpp",
-    "llmserve_attention_f32": "pippppppippiiiiiifiipfpp",
-    "llmserve_attention_tiles": "pippppppippiiiiiifiiipippfpp",
+    "llmserve_attention_generic": "pipipppippiiiiifipfpip",
+    "llmserve_attention_f32": "pippppppippiiiiiifiipfpip",
+    "llmserve_attention_tiles": "pippppppippiiiiiifiiipippfpip",
     "llmserve_attention_portions": "pippppppippiiiiiifiip",
     "llmserve_attention_can_fuse": "i",
     "llmserve_argmax": "ppppiip",
@@ -146,6 +150,7 @@ class GatedLinearWeights:
     both: LinearWeights
     width: int
     activation: str = "silu"
+    limit: float = 0.0  # of "limited_swish"
 
 
 class HipKernels:
@@ -339,7 +344,7 @@ class HipKernels:
             bias = torch.cat(list(biases), dim=0).contiguous() if len(biases) > 1 else biases[0].contiguous()
         return LinearWeights(weight, bias)
 
-    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu") -> GatedLinearWeights:
+    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu", limit: float | None = None) -> GatedLinearWeights:
         """`activation` is the gate's: silu is applied in the epilogue of the product itself, relu too where the
         product has few rows; the others (gelu, gelu_tanh, and relu over many rows) by a kernel of their own
         behind a plain product."""
@@ -347,10 +352,12 @@ class HipKernels:
             raise KernelError(f"gated_linear: no kernel applies the activation {activation!r} (known: {', '.join(_ACTIVATIONS)})")
         if gate.shape != up.shape:
             raise KernelError("gated_linear: gate and up differ in shape")
+        if (activation == "limited_swish") != (limit is not None) or (limit is not None and not limit > 0):
+            raise KernelError("gated_linear: limited_swish, and it alone, has a positive limit")
         if gate.dtype != up.dtype:
             gate, up = gate.float(), up.float()
         both = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
-        return GatedLinearWeights(LinearWeights(both, None), gate.shape[0], activation)
+        return GatedLinearWeights(LinearWeights(both, None), gate.shape[0], activation, float(limit or 0.0))
 
     def _streaming(self, x: torch.Tensor, weights: LinearWeights, gated: bool = False, may_split: bool = False) -> str | None:
         """Which MFMA kernel takes this product: "skinny" (up to 16 rows of x, weights streamed),
@@ -664,9 +671,9 @@ class HipKernels:
             return out
         if weights.activation != "silu":  # no fused epilogue: the product plain, the activation behind it
             both = self.linear(x, weights.both, out_dtype=torch.bfloat16 if self._library(x, weights.both) else torch.float32)
-            status = self._elementwise.llmserve_gate_mul(
+            status = self._elementwise.llmserve_gate_mul_limit(
                 _pointer(both), _is_float(both), _pointer(out), _is_float(out), x.shape[0], weights.width,
-                _ACTIVATIONS[weights.activation], self._stream,
+                _ACTIVATIONS[weights.activation], weights.limit, self._stream,
             )
             _check(status, "gate_mul")
             return out
@@ -804,9 +811,11 @@ class HipKernels:
     def paged_attention(
         self, qkv, layout, batch, cell, scale: float, window: int | None, *,
         score_slopes: torch.Tensor | None = None, soft_cap: float | None = None, sinks: torch.Tensor | None = None,
+        keep_first: int = 0,
     ) -> torch.Tensor:
         """`score_slopes` (float32 [heads]) and `soft_cap` change the scores before the softmax: cap * tanh(score /
-        cap), then minus slope * distance; `sinks` (float32 [heads]) add exp(sink) to a head's denominator.  The
+        cap), then minus slope * distance; `sinks` (float32 [heads]) add exp(sink) to a head's denominator; with
+        `keep_first` a sequence's first so many keys stay visible behind the window, at their own positions.  The
         matrix-core kernels of both precisions take them (in bfloat16 not the forms that fuse the rotation or share
         keys through LDS)."""
         tokens = qkv.shape[0]
@@ -819,15 +828,18 @@ class HipKernels:
             raise KernelError("paged_attention: soft_cap must be positive")
         if sinks is not None and (sinks.dtype != torch.float32 or sinks.shape != (layout.num_heads,)):
             raise KernelError("paged_attention: sinks is one float32 per query head")
+        keep_first = int(keep_first or 0) if window else 0
+        if keep_first < 0 or keep_first != int(getattr(cell.need, "keep_first", 0) or 0):
+            raise KernelError("paged_attention: keep_first is what the cell's pages are kept for")
         out = self._empty((tokens, layout.num_heads * layout.head_dim), qkv.dtype)
         dim = layout.head_dim
-        plain_scores = score_slopes is None and soft_cap is None and sinks is None
+        plain_scores = score_slopes is None and soft_cap is None and sinks is None and not keep_first
         if qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
-            changed = None if plain_scores else (score_slopes, float(soft_cap or 0.0), sinks)
+            changed = None if plain_scores else (score_slopes, float(soft_cap or 0.0), sinks, keep_first)
             self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), changed=changed)
             return out
         if qkv.dtype == torch.float32 and group.page_size % 4 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
-            self._attention_float32(qkv, out, layout, batch, cell, group, scale, int(window or 0), score_slopes, soft_cap, sinks)
+            self._attention_float32(qkv, out, layout, batch, cell, group, scale, int(window or 0), score_slopes, soft_cap, sinks, keep_first)
             return out
         if qkv.dtype == torch.bfloat16:
             why = f"head size {dim} and pages of {group.page_size}"
@@ -836,12 +848,13 @@ class HipKernels:
             _pointer(qkv), layout.width, _pointer(out), _is_float(qkv), _pointer(cell.keys), _pointer(cell.values),
             _pointer(group.block_tables), group.width, _pointer(batch.token_sequence), _pointer(batch.positions),
             tokens, layout.num_heads, layout.num_kv_heads, dim, group.page_size,
-            scale, int(window or 0), _pointer(score_slopes), float(soft_cap or 0.0), _pointer(sinks), self._stream,
+            scale, int(window or 0), _pointer(score_slopes), float(soft_cap or 0.0), _pointer(sinks), keep_first, self._stream,
         )
         _check(status, "paged_attention")
         return out
 
-    def _attention_float32(self, qkv, out, layout, batch, cell, group, scale: float, window: int, score_slopes=None, soft_cap=None, sinks=None) -> None:
+    def _attention_float32(self, qkv, out, layout, batch, cell, group, scale: float, window: int, score_slopes=None, soft_cap=None, sinks=None,
+                           keep_first: int = 0) -> None:
         """The 32-bit path's attention on the matrix cores: an item is 16 (decoding) or 32 columns of one
         request, (token, head) pairs running through the tokens head by head whatever the number of heads; few
         items over long contexts are cut into key splits that a second kernel merges."""
@@ -869,7 +882,7 @@ class HipKernels:
             _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml), _pointer(cell.keys),
             _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work),
             items, column_tiles, tokens, heads, kv_heads, group.page_size, scale, window, splits, _pointer(score_slopes),
-            float(soft_cap or 0.0), _pointer(sinks), self._stream,
+            float(soft_cap or 0.0), _pointer(sinks), keep_first, self._stream,
         )
         _check(status, "paged_attention")
 
@@ -884,7 +897,7 @@ class HipKernels:
         the softmax or a sink in its denominator, which neither `fuse` nor the kernel that shares keys through LDS takes."""
         if changed is not None and fuse is not None:
             raise KernelError("paged_attention: the fused decode form takes plain scores only")
-        slopes, soft_cap, sinks = changed if changed is not None else (None, 0.0, None)
+        slopes, soft_cap, sinks, keep_first = (*changed, 0)[:4] if changed is not None else (None, 0.0, None, 0)
         library = self._attention_library(layout.head_dim)
         heads, kv_heads = layout.num_heads, layout.num_kv_heads
         per_tile = max(1, 16 // (heads // kv_heads))
@@ -1014,7 +1027,7 @@ class HipKernels:
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
                 _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
                 group.page_size, scale, window, splits, (1 if fuse is not None else 0) + (2 if unmerged else 0) + (4 if by_item else 0),
-                _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), _pointer(slopes), soft_cap, _pointer(sinks), self._stream,
+                _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), _pointer(slopes), soft_cap, _pointer(sinks), keep_first, self._stream,
             )
             _check(status, "paged_attention")
             if unmerged and splits > 1:
@@ -1199,16 +1212,19 @@ class HipKernels:
         _check(status, "route")
         return chosen, weights
 
-    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str, gates: list[torch.Tensor] | None = None):
+    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str, gates: list[torch.Tensor] | None = None,
+                        limit: float | None = None):
         """The experts' weights stacked: ([experts, size, hidden], [experts, hidden, size], activation, gated).  With `gates`
         an expert's gate and up rows alternate (gate_0, up_0, gate_1, ...: [experts, 2 size, hidden]), so that a row of the
         first product holds every gate beside its up."""
         if activation not in _ACTIVATIONS:
             raise KernelError(f"experts: no kernel applies the activation {activation!r} (known: {', '.join(_ACTIVATIONS)})")
+        if (activation == "limited_swish") != (limit is not None) or (limit is not None and (gates is None or not limit > 0)):
+            raise KernelError("experts: limited_swish, and it alone, has a positive limit, and gates an expert")
         if gates is None:
             return torch.stack(list(ups)).contiguous(), torch.stack(list(downs)).contiguous(), activation, False
         both = torch.stack([torch.stack([gate, up], dim=1).reshape(2 * up.shape[0], up.shape[1]) for gate, up in zip(gates, ups)])
-        return both.contiguous(), torch.stack(list(downs)).contiguous(), activation, True
+        return both.contiguous(), torch.stack(list(downs)).contiguous(), (activation, float(limit)) if limit is not None else activation, True
 
     def expert_feed_forward(self, x, experts, chosen, weights, shared=None, gates=None, gate_column: int = 0) -> torch.Tensor:
         """sum over a token's chosen experts of weight * down(act(up x)), float32 [T, hidden].  The (token, choice)
@@ -1216,6 +1232,7 @@ class HipKernels:
         kernel adds each token's rows up in the order of its choices; with `shared` (float32 [T, hidden]) it adds
         sigmoid(gates[:, gate_column]) * shared as well."""
         ups, downs, activation, gated = experts
+        activation, limit = activation if isinstance(activation, tuple) else (activation, 0.0)
         tokens, top = chosen.shape
         count, size, hidden = ups.shape  # (gated: `size` counts gate and up rows, twice the experts' width)
         if x.dtype != ups.dtype or x.shape != (tokens, hidden):
@@ -1235,7 +1252,8 @@ class HipKernels:
         _check(library.llmserve_sort_pairs(_pointer(chosen), pairs, count, _pointer(place), _pointer(order), _pointer(tiles), capacity, tile_rows, self._stream), "experts: sort")
         # the matrix-core kernels gate their result themselves (act(gate) * up of neighbouring columns); behind the others a
         # kernel of its own does
-        fused = gated and bool(library.llmserve_expert_product_gates(_is_float(x), hidden, tile_rows))
+        # (the gate with a limit is a function of gate and up both: the kernel behind the product applies it)
+        fused = gated and activation != "limited_swish" and bool(library.llmserve_expert_product_gates(_is_float(x), hidden, tile_rows))
         code = _ACTIVATIONS[activation] + _GATED_RESULT if fused else -1 if gated else _ACTIVATIONS[activation]
         inner = self._empty((pairs, width if fused else size), x.dtype)
         _check(library.llmserve_expert_product(
@@ -1244,8 +1262,8 @@ class HipKernels:
         if gated and not fused:
             both = inner
             inner = self._empty((pairs, width), x.dtype)
-            _check(self._elementwise.llmserve_gate_mul(
-                _pointer(both), _is_float(both), _pointer(inner), _is_float(inner), pairs, width, _ACTIVATIONS[activation], self._stream), "experts: gate")
+            _check(self._elementwise.llmserve_gate_mul_limit(
+                _pointer(both), _is_float(both), _pointer(inner), _is_float(inner), pairs, width, _ACTIVATIONS[activation], limit, self._stream), "experts: gate")
         size = width
         rows = self._empty((pairs, hidden), torch.float32)
         _check(library.llmserve_expert_product(
@@ -1383,6 +1401,45 @@ class HipKernels:
         )
         _check(status, "add_normed")
         return hidden if out is None else out
+
+    def add_normed_norm(self, hidden, update, weight, eps: float, next_weight, next_eps: float) -> torch.Tensor:
+        rows, width = hidden.shape
+        if hidden.dtype != torch.float32 or update.dtype != torch.float32 or update.shape[-2:] != (rows, width) or weight.shape != (width,) \
+                or next_weight.shape != (width,):
+            raise KernelError("add_normed_norm: a float32 stream, float32 rows (or parts of them) of its shape and two weights as long as a row")
+        out = self._empty((rows, width), self.dtype)
+        parts = 1 if update.ndim == 2 else update.shape[0]
+        status = self._library_of("heads").llmserve_add_normed_norm(
+            _pointer(hidden), _pointer(update), parts, _pointer(weight), _is_float(weight), eps, _pointer(next_weight), _is_float(next_weight),
+            next_eps, _pointer(out), _is_float(out), rows, width, self._stream,
+        )
+        _check(status, "add_normed_norm")
+        return out
+
+    def rotate_heads(self, x, first: int, head_stride: int, heads: int, table, dims: int, pairing: str, scale: float = 1.0) -> torch.Tensor:
+        tokens = x.shape[0]
+        if dims and (pairing not in ("adjacent", "half") or table is None or table.dtype != torch.float32 or table.shape != (tokens, dims // 2, 2)):
+            raise KernelError("rotate_heads: pairs that are adjacent or halves apart, and a float32 table entry for every pair of every token")
+        status = self._library_of("heads").llmserve_rotate_heads(
+            _pointer(x), _is_float(x), tokens, x.shape[1], first, head_stride, heads, _pointer(table if dims else None), dims,
+            _PAIRINGS[pairing] if dims else 0, float(scale), self._stream,
+        )
+        _check(status, "rotate_heads")
+        return x
+
+    def add_rows(self, hidden, delta, other, vector) -> torch.Tensor:
+        rows, width = hidden.shape
+        for name, tensor, shape in (("delta", delta, None), ("other", other, (rows, width)), ("vector", vector, (width,))):
+            if tensor is not None and (tensor.dtype != torch.float32 or (shape is not None and tensor.shape != shape)):
+                raise KernelError(f"add_rows: {name} is float32 and fits the stream")
+        if hidden.dtype != torch.float32 or (delta is not None and delta.shape[-2:] != (rows, width)):
+            raise KernelError("add_rows: a float32 stream and rows (or parts of them) of its shape")
+        parts = 1 if delta is None or delta.ndim == 2 else delta.shape[0]
+        status = self._library_of("heads").llmserve_add_rows(
+            _pointer(hidden), _pointer(delta), parts, _pointer(other), _pointer(vector), rows, width, self._stream
+        )
+        _check(status, "add_rows")
+        return hidden
 
     def assemble_heads(self, x, q_first: int, k_first: int, v_first: int, heads: int, kv_heads: int, dim: int, vdim: int, width: int,
                        norm, q_weight, k_weight, eps: float, table, rot_dims: int, other=None, other_first: int = 0, blend: float = 0.0,

@@ -34,9 +34,11 @@ class Kernels(Protocol):
     def prepare_linear(self, weights: list[torch.Tensor], biases: list[torch.Tensor] | None) -> Any:
         """Concatenates [N_i, K] weights (and biases) along N into whatever layout `linear` wants."""
 
-    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu") -> Any:
+    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu", limit: float | None = None) -> Any:
         """Gate and up weights [I, K] in whatever layout `gated_linear` wants; `activation` is the gate's
-        (silu, gelu, gelu_tanh, relu), and one the library has no kernel for is refused here, by name."""
+        (silu, gelu, gelu_tanh, relu), and one the library has no kernel for is refused here, by name.
+        "limited_swish" is a function of gate and up both and has a `limit`: g = min(gate, limit), u = clamp(up,
+        -limit, limit), and the result is g * sigmoid(1.702 g) * (u + 1)."""
 
     def linear(
         self, x: torch.Tensor, weights: Any, out_dtype: torch.dtype | None = None, *, partial: bool = False
@@ -56,13 +58,16 @@ class Kernels(Protocol):
     def paged_attention(
         self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any, scale: float, window: int | None, *,
         score_slopes: torch.Tensor | None = None, soft_cap: float | None = None, sinks: torch.Tensor | None = None,
+        keep_first: int = 0,
     ) -> torch.Tensor:
         """Attention of the q heads of `qkv` over the cell's pages -> [T, heads * head_dim].
         Before the softmax a score s of a query at position p for a key at position k may be changed,
         for encodings and models that want it (Qwen2 wants neither): with `soft_cap`, to
         soft_cap * tanh(s / soft_cap); with `score_slopes` (float32, one per query head), by
         - slope * (p - k) after that.  With `sinks` (float32, one per query head) the softmax's denominator
-        has exp(sink) more, once, with no value to it.  A library refuses what it cannot compute."""
+        has exp(sink) more, once, with no value to it.  With `keep_first` (and a window) a query at p sees the keys at
+        k <= p with p - k < window or k < keep_first: a sequence's first keys stay visible, at their own positions (the
+        cell's need says the same, so their pages are never given back).  A library refuses what it cannot compute."""
 
     def rotate_store_attend(
         self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any,
@@ -163,6 +168,24 @@ class Kernels(Protocol):
         """`hidden += u * rsqrt(mean(u^2) + eps) * weight` in place, u the float32 rows of `update` (its parts added
         first); -> the new rows in the run dtype (in a float32 run the stream itself)."""
 
+    def add_normed_norm(
+        self, hidden: torch.Tensor, update: torch.Tensor, weight: torch.Tensor, eps: float, next_weight: torch.Tensor, next_eps: float,
+    ) -> torch.Tensor:
+        """`add_normed`, and then the norm before the next sublayer in the same pass over the row: -> the new rows *
+        rsqrt(mean(new rows^2) + next_eps) * next_weight in the run dtype."""
+
+    def rotate_heads(
+        self, x: torch.Tensor, first: int, head_stride: int, heads: int, table: torch.Tensor | None, dims: int, pairing: str, scale: float = 1.0,
+    ) -> torch.Tensor:
+        """In place, for `heads` heads of `head_stride` columns from column `first` of x's rows (float32 or the run
+        dtype): the first `dims` columns of a head turn in pairs (`pairing` "adjacent": (2i, 2i + 1); "half": (i, i +
+        dims / 2)) by the token's row of `table` (float32 [T, dims / 2, 2], cos and sin), and the whole head is multiplied
+        by `scale`; float32 arithmetic."""
+
+    def add_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None, other: torch.Tensor | None, vector: torch.Tensor | None) -> torch.Tensor:
+        """`hidden += delta (its parts added in order) + other + vector` in place, float32: `other` rows of the stream's
+        shape, `vector` one row for all; any of the three may be None.  -> hidden."""
+
     def assemble_heads(
         self, x: torch.Tensor, q_first: int, k_first: int, v_first: int, heads: int, kv_heads: int, dim: int, vdim: int,
         width: int, norm: str | None, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
@@ -188,7 +211,7 @@ class Kernels(Protocol):
     ) -> torch.Tensor:
         """q, k (heads of dim) and v (heads of vdim) are act of x's columns from q_first, k_first, v_first.  Per request
         and head, token by token: S = decay_h S + k v^T; o = S^T q.  `state` float32 [slots, heads, dim, vdim] holds S
-        and is updated; decays float32 [heads].  -> float32 [T, heads * vdim]."""
+        and is updated; decays float32 [heads]; act is "silu" or "none"; x in the run dtype or float32.  -> float32 [T, heads * vdim]."""
 
     def soft_cap(self, logits: torch.Tensor, cap: float) -> torch.Tensor:
         """cap * tanh(logits / cap), in place (float32)."""
@@ -204,8 +227,11 @@ class Kernels(Protocol):
         neighbours (a group's score is its largest); -> (int32 [T, top] experts, float32 [T, top] weights = scale * s of the
         chosen, with `renormalise` scale * s / (sum of the chosen s + 1e-20))."""
 
-    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str, gates: list[torch.Tensor] | None = None) -> Any:
-        """With `gates` an expert is down(act(gate x) * (up x)), else down(act(up x))."""
+    def prepare_experts(
+        self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str, gates: list[torch.Tensor] | None = None, limit: float | None = None,
+    ) -> Any:
+        """With `gates` an expert is down(act(gate x) * (up x)), else down(act(up x)); "limited_swish" (with `gates` and a
+        `limit`) is the function of gate and up that `prepare_gated_linear` describes."""
 
     def expert_feed_forward(
         self, x: torch.Tensor, experts: Any, chosen: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None = None,

@@ -1,3 +1,3 @@
-from . import dafutar, katenex, qwen2, sozavik  # register Dafutar, Katenex, Qwen2ForCausalLM and Sozavik
+from . import dafutar, katenex, qwen2, sozavik, vagozen  # register Dafutar, Katenex, Qwen2ForCausalLM, Sozavik and Vagozen
 
-__all__ = ["dafutar", "katenex", "qwen2", "sozavik"]
+__all__ = ["dafutar", "katenex", "qwen2", "sozavik", "vagozen"]

@@ -20,8 +20,8 @@ from .norm import LayerNorm, LayerNormSpec, RMSNorm, RMSNormSpec
 from .position import HeadLayout, LinearScaling, NoPositionSpec, PositionEncoding, Rotary, RotarySpec, WavelengthScaling, YarnScaling, rotary_frequencies
 from .attention import Attention, AttentionSpec, Mixer
 from .feed_forward import FeedForward, GatedMLP, GatedMLPSpec
-from .block import Block, OutputNormBlock, OutputNormBlockSpec, PreNormBlock, PreNormBlockSpec
-from .model import DecoderModel, JoinedPass, JoinedPassSpec, LayerDefinition, LayerRun, ModelSpec, NamedPart, SoftCap, SoftCapSpec
+from .block import Block, OutputNormBlock, OutputNormBlockSpec, PendingNormed, PreNormBlock, PreNormBlockSpec, SandwichBlock, SandwichBlockSpec
+from .model import AddedPass, AddedPassSpec, DecoderModel, JoinedPass, JoinedPassSpec, LayerDefinition, LayerRun, ModelSpec, NamedPart, SoftCap, SoftCapSpec
 from .latent_attention import LatentAttention, LatentAttentionSpec
 from .delta import GatedDelta, GatedDeltaSpec
 from .experts import RoutedExperts, RoutedExpertsSpec

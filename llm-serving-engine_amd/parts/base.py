@@ -58,9 +58,11 @@ class CacheNeed:
 
 class PagedNeed(CacheNeed):
     """An entry per token.  A subclass has a field `window` (keys at most that are ever read again, None:
-    all) and says what one page holds."""
+    all), may have a field `keep_first` (so many entries at a request's start are read for ever, whatever the
+    window), and says what one page holds."""
 
     window: int | None = None
+    keep_first: int = 0
 
     def page_fields(self, page_size: int) -> dict[str, tuple[int, ...]]:
         """name -> shape of ONE page of that field.  The cache keeps each field as a tensor
@@ -94,6 +96,7 @@ class PagedKeyValue(PagedNeed):
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    keep_first: int = 0
 
     def page_fields(self, page_size: int) -> dict[str, tuple[int, ...]]:
         width = key_piece_width(self.head_dim)

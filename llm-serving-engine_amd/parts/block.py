@@ -112,3 +112,117 @@ class OutputNormBlock(PreNormBlock):
             rows = self.feed_forward_norm.add_normed(hidden, self.feed_forward.forward(rows, batch))
         batch.computed["stream rows"] = (hidden, rows)
         return None
+
+
+@dataclass
+class PendingNormed:
+    """What a sublayer leaves for the stream when its result is normed before it is added: `hidden += update *
+    rsqrt(mean(update^2) + eps) * weight` is still to do (`update` float32 rows, or partial sums of them).  The next
+    block of the same kind does it in the kernel that norms the stream for its mixer; anyone else calls `settle`."""
+
+    update: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+    kernels: Any
+
+    def settle(self, hidden: torch.Tensor) -> None:
+        self.kernels.add_normed(hidden, self.update, self.weight, self.eps)
+        return None
+
+
+@dataclass(frozen=True)
+class SandwichBlockSpec:
+    """h += scale1 * norm1b(mixer(norm1(h))); h += scale2 * norm2b(feed_forward(norm2(h))): a norm before and one behind
+    every sublayer, and a learned vector (`*_scale_name`, as long as a row; None: none) on what is added.  A layer
+    without a feed-forward has `feed_forward` None.  The `*_name` fields are the prefixes (the scales' the names) of
+    the members' tensors below the layer's own prefix."""
+
+    mixer_norm: Any
+    mixer: Any
+    mixer_out_norm: Any
+    feed_forward_norm: Any
+    feed_forward: Any
+    feed_forward_out_norm: Any
+    mixer_norm_name: str = "norm1."
+    mixer_name: str = "mix."
+    mixer_out_norm_name: str = "norm1b."
+    feed_forward_norm_name: str = "norm2."
+    feed_forward_name: str = "mlp."
+    feed_forward_out_norm_name: str = "norm2b."
+    mixer_scale_name: str | None = "ls1"
+    feed_forward_scale_name: str | None = "ls2"
+    kind: str = "sandwich"
+
+
+@BLOCKS.register("sandwich")
+class SandwichBlock(Block):
+    """The norms are RMS norms with a weight.  The vector on a sublayer's result is multiplied into the weight of the
+    norm behind the sublayer when the block is built (float32), so it costs nothing in a step.  The norm behind a
+    sublayer, the add and the norm before the next sublayer are one kernel: the stream is read and written once a
+    sublayer.  What the last sublayer leaves is handed on as a `PendingNormed`."""
+
+    accepts_pending_normed = True
+
+    @classmethod
+    def _members(cls, spec: SandwichBlockSpec):
+        members = [
+            (spec.mixer_norm_name, NORMS, spec.mixer_norm), (spec.mixer_name, MIXERS, spec.mixer),
+            (spec.mixer_out_norm_name, NORMS, spec.mixer_out_norm),
+        ]
+        if spec.feed_forward is not None:
+            members += [
+                (spec.feed_forward_norm_name, NORMS, spec.feed_forward_norm), (spec.feed_forward_name, FEED_FORWARDS, spec.feed_forward),
+                (spec.feed_forward_out_norm_name, NORMS, spec.feed_forward_out_norm),
+            ]
+        return tuple(members)
+
+    @classmethod
+    def tensors(cls, spec: SandwichBlockSpec) -> dict[str, TensorSpec]:
+        found: dict[str, TensorSpec] = {}
+        for name, registry, member in cls._members(spec):
+            found.update(prefixed(registry.tensors(member), name))
+        if spec.mixer_scale_name is not None:
+            found[spec.mixer_scale_name] = TensorSpec((spec.mixer_out_norm.size,), role="norm")
+        if spec.feed_forward is not None and spec.feed_forward_scale_name is not None:
+            found[spec.feed_forward_scale_name] = TensorSpec((spec.feed_forward_out_norm.size,), role="norm")
+        return found
+
+    @classmethod
+    def cache_need(cls, spec: SandwichBlockSpec) -> CacheNeed:
+        return MIXERS.cache_need(spec.mixer)
+
+    def __init__(self, spec: SandwichBlockSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        built = [registry.build(member, under(tensors, name), kernels) for name, registry, member in self._members(spec)]
+        for norm in (built[0], built[2], *(built[3::2])):
+            if not hasattr(norm, "weight") or hasattr(norm, "bias"):
+                raise ValueError("sandwich block: its norms are RMS norms with a weight")
+        self.mixer_norm, self.mixer = built[0], built[1]
+
+        def scaled(norm, name):
+            weight = norm.weight.float()
+            return (weight * tensors[name].float() if name is not None else weight).contiguous()
+
+        self.mixer_out = scaled(built[2], spec.mixer_scale_name)
+        self.mixer_out_eps = spec.mixer_out_norm.eps
+        self.feed_forward_norm = self.feed_forward = self.feed_forward_out = None
+        if spec.feed_forward is not None:
+            self.feed_forward_norm, self.feed_forward = built[3], built[4]
+            self.feed_forward_out = scaled(built[5], spec.feed_forward_scale_name)
+            self.feed_forward_out_eps = spec.feed_forward_out_norm.eps
+        self.replayable = all(part.replayable for part in built)
+
+    def forward(self, hidden, delta, batch, cell):
+        kernels = self.kernels
+        if isinstance(delta, PendingNormed):
+            normed = kernels.add_normed_norm(hidden, delta.update, delta.weight, delta.eps, self.mixer_norm.weight, self.mixer_norm.spec.eps)
+        else:
+            normed = self.mixer_norm.forward(hidden, delta)
+        mixed = self.mixer.forward(normed, batch, cell)
+        if self.feed_forward is None:
+            return PendingNormed(mixed, self.mixer_out, self.mixer_out_eps, kernels)
+        normed = kernels.add_normed_norm(
+            hidden, mixed, self.mixer_out, self.mixer_out_eps, self.feed_forward_norm.weight, self.feed_forward_norm.spec.eps
+        )
+        fed = self.feed_forward.forward(normed, batch)
+        return PendingNormed(fed, self.feed_forward_out, self.feed_forward_out_eps, kernels)

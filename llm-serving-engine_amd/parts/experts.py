@@ -18,7 +18,10 @@ class RoutedExpertsSpec:
     experts of the `keep_groups` best of `groups` equal groups of neighbours (a group's score is its largest), and
     weighted by its score times `route_scale`; with `renormalise` the chosen scores are divided by their sum (+ 1e-20)
     first.  `shared_size` (None: none) is the width of an expert that every token uses, of the same form, scaled by
-    sigmoid of a gate of its own (`shared_gate` False: added as it is)."""
+    sigmoid of a gate of its own (`shared_gate` False: added as it is).  `router_bias`: the router's logits have a bias
+    (`router.b`), part of the float32 product.  `limit`: of the activation "limited_swish" (g = min(gate, limit), u =
+    clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1)).  A softmax over the chosen logits alone is `scoring`
+    "softmax" with `renormalise`: the sum over all experts cancels."""
 
     hidden_size: int
     num_experts: int
@@ -35,6 +38,8 @@ class RoutedExpertsSpec:
     keep_groups: int = 1
     renormalise: bool = False
     shared_gate: bool = True
+    router_bias: bool = False
+    limit: float | None = None
     kind: str = "routed_experts"
 
 
@@ -48,6 +53,8 @@ class RoutedExperts(FeedForward):
     @classmethod
     def tensors(cls, spec: RoutedExpertsSpec) -> dict[str, TensorSpec]:
         found = {"router": TensorSpec((spec.num_experts, spec.hidden_size))}
+        if spec.router_bias:
+            found["router.b"] = TensorSpec((spec.num_experts,), role="bias")
         if spec.correction:
             found["correction"] = TensorSpec((spec.num_experts,), role="bias")
         for index in range(spec.num_experts):
@@ -72,13 +79,18 @@ class RoutedExperts(FeedForward):
             raise ValueError("routed experts: equal groups, between one and all of them kept, with room for a token's experts")
         shared = spec.shared_size is not None
         # the shared expert's gate is one more row of the router's product
-        self.router = kernels.prepare_linear([tensors["router"]] + ([tensors["shared.sg"]] if shared and spec.shared_gate else []), None)
+        gate_row = [tensors["shared.sg"]] if shared and spec.shared_gate else []
+        biases = None
+        if spec.router_bias:
+            biases = [tensors["router.b"]] + [torch.zeros((1,), dtype=tensors["router.b"].dtype, device=tensors["router.b"].device) for _ in gate_row]
+        self.router = kernels.prepare_linear([tensors["router"]] + gate_row, biases)
         self.correction = kernels.to_device(tensors["correction"].float().contiguous()) if spec.correction else None
         self.experts = kernels.prepare_experts(
             [tensors[f"e{index}.up"] for index in range(spec.num_experts)],
             [tensors[f"e{index}.down"] for index in range(spec.num_experts)],
             spec.activation,
             gates=[tensors[f"e{index}.gate"] for index in range(spec.num_experts)] if spec.gated else None,
+            **({"limit": spec.limit} if spec.limit is not None else {}),
         )
         self.shared_up = self.shared_down = None
         if shared:

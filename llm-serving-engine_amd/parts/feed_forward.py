@@ -26,6 +26,8 @@ class GatedMLPSpec:
     kind: str = "gated_mlp"
     # the tensors' names below the part's prefix: gate, up, down
     names: tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
+    # of the activation "limited_swish": g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1)
+    limit: float | None = None
 
 
 @FEED_FORWARDS.register("gated_mlp")
@@ -46,7 +48,10 @@ class GatedMLP(FeedForward):
         super().__init__(spec, tensors, kernels)
         # the kernel library says which activations it has, and refuses another by name
         gate, up, down = spec.names
-        self.gate_up = kernels.prepare_gated_linear(tensors[gate], tensors[up], spec.activation)
+        if spec.limit is None:
+            self.gate_up = kernels.prepare_gated_linear(tensors[gate], tensors[up], spec.activation)
+        else:
+            self.gate_up = kernels.prepare_gated_linear(tensors[gate], tensors[up], spec.activation, limit=spec.limit)
         self.down = kernels.prepare_linear([tensors[down]], None)
 
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:

@@ -130,11 +130,20 @@ class DecoderModel:
         embedded = hidden.clone() if self.pass_entry is not None else None  # the layers add into `hidden` in place
         delta = None
         for index, (run, cell) in enumerate(zip(self.spec.run_order, cells)):
+            layer = self.layers[run.layer]
+            # what a block left to do in a form of its own (a result that is normed before it is added) is done here
+            # unless the next block takes it as it is
+            if hasattr(delta, "settle") and (run.enters is not None or not getattr(layer, "accepts_pending_normed", False)):
+                delta = delta.settle(hidden)
             if run.enters is not None:
                 hidden, delta = self.pass_entry.forward(hidden, delta, embedded, batch, run.enters), None
-            delta = self.layers[run.layer].forward(hidden, delta, batch, cell)
+            delta = layer.forward(hidden, delta, batch, cell)
             if self.observer is not None:
+                if hasattr(delta, "settle"):
+                    delta = delta.settle(hidden)
                 self.observer(index, hidden, delta)
+        if hasattr(delta, "settle"):
+            delta = delta.settle(hidden)
         return hidden, delta
 
     def forward_without_logits(self, batch, cells: list) -> None:
@@ -198,6 +207,42 @@ class JoinedPass:
     def forward(self, hidden, delta, embedded, batch, number: int):
         both = self.kernels.join_rows(hidden, delta, embedded)  # [T, 2 hidden] in the run dtype
         return self.kernels.linear(both, self.products[number], out_dtype=torch.float32)
+
+
+@dataclass(frozen=True)
+class AddedPassSpec:
+    """x <- x + x0 (every pass but the first) + step[t] at the start of pass t, x0 the embedded stream; `passes` is how
+    many there are.  `step_name` [passes, hidden] below the part's prefix."""
+
+    hidden_size: int
+    passes: int
+    step_name: str = "step"
+    kind: str = "added_pass"
+
+
+@PASS_PARTS.register("added_pass")
+class AddedPass:
+    """The stream that enters a pass is the stream so far plus a vector of the pass and, from the second pass on, plus
+    the embedded stream: one kernel, in place, in float32."""
+
+    replayable = True
+
+    @classmethod
+    def tensors(cls, spec: AddedPassSpec) -> dict[str, TensorSpec]:
+        return {spec.step_name: TensorSpec((spec.passes, spec.hidden_size), role="bias")}
+
+    @classmethod
+    def cache_need(cls, spec: AddedPassSpec) -> None:
+        return None
+
+    def __init__(self, spec: AddedPassSpec, tensors, kernels) -> None:
+        self.spec = spec
+        self.kernels = kernels
+        steps = tensors[spec.step_name]
+        self.steps = [steps[index].float().contiguous() for index in range(spec.passes)]
+
+    def forward(self, hidden, delta, embedded, batch, number: int):
+        return self.kernels.add_rows(hidden, delta, embedded if number > 0 else None, self.steps[number])
 
 
 @dataclass(frozen=True)

@@ -11,12 +11,15 @@ from .base import NORMS, Part, TensorSpec
 
 @dataclass(frozen=True)
 class RMSNormSpec:
-    """`weight_name` is the tensor's name below the part's prefix (a model whose files call it otherwise says so)."""
+    """`weight_name` is the tensor's name below the part's prefix (a model whose files call it otherwise says so).
+    `weight_scale` multiplies the weight (float32) when the part is built: a constant that a model puts on the normed
+    rows (a scale of the logits behind the last norm) costs nothing that way."""
 
     size: int
     eps: float
     weight_name: str = "weight"
     kind: str = "rmsnorm"
+    weight_scale: float = 1.0
 
 
 @NORMS.register("rmsnorm")
@@ -32,6 +35,8 @@ class RMSNorm(Part):
     def __init__(self, spec: RMSNormSpec, tensors, kernels) -> None:
         super().__init__(spec, tensors, kernels)
         self.weight = tensors[spec.weight_name]
+        if spec.weight_scale != 1.0:
+            self.weight = (self.weight.float() * float(spec.weight_scale)).contiguous()
 
     def forward(self, hidden: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
         """Adds `delta` into `hidden` (in place) and returns the normed rows in the run dtype."""

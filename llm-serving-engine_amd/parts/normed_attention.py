@@ -26,7 +26,9 @@ class NormedAttentionSpec:
     `soft_cap`: scores become cap * tanh(score / cap).  `sink`: a learned number a head whose exponential is added
     once to the softmax's denominator.  `gate`: head h's result times sigmoid of row h of a product of the mixer's input.
     `values`: None, "give" (the step's values are shown to later layers under `values_name`) or "take" (v <- (1 - a) v
-    + a v_given with the learned number a; the blended v is what is cached)."""
+    + a v_given with the learned number a; the blended v is what is cached).
+    `keep_first`: under a window, the first so many tokens of a sequence stay visible to every later query, at their
+    own positions (a query at p sees the keys at j <= p with p - j < window or j < keep_first)."""
 
     hidden_size: int
     num_heads: int
@@ -47,6 +49,7 @@ class NormedAttentionSpec:
     gate: bool = False
     values: str | None = None
     values_name: str = "values"
+    keep_first: int = 0
     kind: str = "normed_attention"
 
     @property
@@ -90,7 +93,7 @@ class NormedAttention(Mixer):
 
     @classmethod
     def cache_need(cls, spec: NormedAttentionSpec) -> PagedKeyValue:
-        return PagedKeyValue(spec.num_kv_heads, spec.head_width, spec.window)
+        return PagedKeyValue(spec.num_kv_heads, spec.head_width, spec.window, spec.keep_first if spec.window is not None else 0)
 
     def __init__(self, spec: NormedAttentionSpec, tensors, kernels) -> None:
         super().__init__(spec, tensors, kernels)
@@ -102,6 +105,9 @@ class NormedAttention(Mixer):
             raise ValueError("normed attention: pairing is 'adjacent' or 'half'")
         if spec.rot_dims % 2 or spec.rot_dims > spec.dim:
             raise ValueError("normed attention: the rotated dimensions are an even number within dim")
+        if spec.keep_first < 0:
+            raise ValueError("normed attention: keep_first counts tokens")
+        self.keep_first = spec.keep_first if spec.window is not None else 0
         heads, width = spec.num_heads, spec.head_width
         self.layout = HeadLayout(heads, spec.num_kv_heads, width)
         names = ["q", "k", "v"] + (["g"] if spec.gate else [])
@@ -143,7 +149,7 @@ class NormedAttention(Mixer):
                 raise RuntimeError("normed attention: no earlier layer of this step gave values of this size")
         table = kernels.rotary_table(batch, self.frequencies, self.magnitude) if spec.rot_dims else None
         # per token the heads' queries, keys and values as the attention reads them: normed, turned, blended, widened
-        plain = spec.soft_cap is None and self.sinks is None and not spec.gate
+        plain = spec.soft_cap is None and self.sinks is None and not spec.gate and not self.keep_first
         rows = kernels.assemble_heads(
             projected, 0, q_size, q_size + k_size, spec.num_heads, spec.num_kv_heads, spec.dim, spec.vdim, spec.head_width,
             spec.norm, self.q_norm, self.k_norm, spec.eps, table, spec.rot_dims,
@@ -153,7 +159,9 @@ class NormedAttention(Mixer):
         )
         if plain:
             return kernels.rotate_store_attend(rows, self.layout, batch, cell, None, "none", spec.scale, spec.window, project=self.out)
-        mixed = kernels.paged_attention(rows, self.layout, batch, cell, spec.scale, spec.window, soft_cap=spec.soft_cap, sinks=self.sinks)
+        mixed = kernels.paged_attention(
+            rows, self.layout, batch, cell, spec.scale, spec.window, soft_cap=spec.soft_cap, sinks=self.sinks, keep_first=self.keep_first,
+        )
         if spec.gate:
             kernels.scale_heads(mixed, spec.num_heads, spec.head_width, projected, q_size + k_size + v_size, "sigmoid")
         return kernels.linear(mixed, self.out, out_dtype=torch.float32, partial=True)

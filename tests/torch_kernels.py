@@ -20,6 +20,11 @@ class _Linear:
     bias: torch.Tensor | None
 
 
+def _limited_swish(gate, up, limit):
+    g = gate.clamp(max=limit)
+    return g * torch.sigmoid(1.702 * g) * (up.clamp(-limit, limit) + 1.0)
+
+
 class TorchKernels:
     def __init__(self, dtype: torch.dtype = torch.float32) -> None:
         self.device = torch.device("cpu")
@@ -46,9 +51,13 @@ class TorchKernels:
         bias = torch.cat([b.float() for b in biases], dim=0) if biases else None
         return _Linear(weight, bias)
 
-    def prepare_gated_linear(self, gate, up, activation="silu"):
+    def prepare_gated_linear(self, gate, up, activation="silu", limit=None):
         acts = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "relu": torch.relu,
                 "gelu_tanh": lambda z: torch.nn.functional.gelu(z, approximate="tanh")}
+        if activation == "limited_swish":
+            if limit is None or not limit > 0:
+                raise ValueError("gated_linear: limited_swish has a positive limit")
+            return (_Linear(gate.float(), None), _Linear(up.float(), None), lambda g, u: _limited_swish(g, u, float(limit)), True)
         if activation not in acts:
             raise ValueError(f"gated_linear: no activation {activation!r}")
         return (_Linear(gate.float(), None), _Linear(up.float(), None), acts[activation])
@@ -62,6 +71,8 @@ class TorchKernels:
     def gated_linear(self, x, weights):
         gate = x.float() @ weights[0].weight.T
         up = x.float() @ weights[1].weight.T
+        if len(weights) > 3:  # a function of gate and up both
+            return weights[2](gate, up).to(self.dtype)
         return (weights[2](gate) * up).to(self.dtype)
 
     def rotate_and_store(self, qkv, layout, batch, cell, inverse_frequencies, pairing):
@@ -88,7 +99,7 @@ class TorchKernels:
             cell.put_key_rows(pages, offsets, view[:, heads : heads + kv_heads])  # pages are [kv, dim / w, offset, w]
             cell.put_value_rows(pages, offsets, view[:, heads + kv_heads :])  # pages are [kv, offset / v, dim, v]
 
-    def paged_attention(self, qkv, layout, batch, cell, scale, window, *, score_slopes=None, soft_cap=None, sinks=None):
+    def paged_attention(self, qkv, layout, batch, cell, scale, window, *, score_slopes=None, soft_cap=None, sinks=None, keep_first=0):
         tokens = qkv.shape[0]
         heads, kv_heads, dim = layout.num_heads, layout.num_kv_heads, layout.head_dim
         queries = qkv.view(tokens, heads + 2 * kv_heads, dim)[:, :heads].float()
@@ -100,6 +111,8 @@ class TorchKernels:
             for position in range(chunk.start, chunk.start + chunk.count):
                 first = 0 if window is None else max(0, position - window + 1)
                 where = torch.arange(first, position + 1)
+                if keep_first and first > 0:  # the sequence's first tokens stay visible, at their own positions
+                    where = torch.cat([torch.arange(0, min(keep_first, first)), where])
                 pages = table[where // group.page_size]
                 assert (pages >= 0).all(), "attention reads a page that was given back"
                 keys = cell.key_rows(pages, where % group.page_size).float()  # [n, kv, D]
@@ -327,10 +340,36 @@ class TorchKernels:
         x.copy_((x.float().view(x.shape[0], heads, width) * gate[:, :, None]).reshape(x.shape).to(x.dtype))
         return x
 
-    def decay_attention(self, x, q_first, k_first, v_first, heads, dim, vdim, decays, activation, batch, state):
-        assert activation == "silu"
+    def rotate_heads(self, x, first, head_stride, heads, table, dims, pairing, scale=1.0):
         tokens = x.shape[0]
-        act = torch.nn.functional.silu
+        for head in range(heads):
+            part = x[:, first + head * head_stride : first + (head + 1) * head_stride].float()
+            if dims:
+                cos, sin = table[:, :, 0], table[:, :, 1]
+                one, two = (slice(0, dims, 2), slice(1, dims, 2)) if pairing == "adjacent" else (slice(0, dims // 2), slice(dims // 2, dims))
+                a, b = part[:, one].clone(), part[:, two].clone()
+                part[:, one] = a * cos - b * sin
+                part[:, two] = b * cos + a * sin
+            x[:, first + head * head_stride : first + (head + 1) * head_stride] = (part * scale).to(x.dtype)
+        return x
+
+    def add_normed_norm(self, hidden, update, weight, eps, next_weight, next_eps):
+        self.add_normed(hidden, update, weight, eps)
+        return self.add_rms_norm(hidden, None, next_weight, next_eps)
+
+    def add_rows(self, hidden, delta, other, vector):
+        if delta is not None:
+            hidden += delta if delta.ndim == 2 else delta.sum(0)
+        if other is not None:
+            hidden += other
+        if vector is not None:
+            hidden += vector.float()
+        return hidden
+
+    def decay_attention(self, x, q_first, k_first, v_first, heads, dim, vdim, decays, activation, batch, state):
+        assert activation in ("silu", "none")
+        tokens = x.shape[0]
+        act = torch.nn.functional.silu if activation == "silu" else (lambda z: z)
         q = act(x[:, q_first : q_first + heads * dim].float()).view(tokens, heads, dim)
         k = act(x[:, k_first : k_first + heads * dim].float()).view(tokens, heads, dim)
         v = act(x[:, v_first : v_first + heads * vdim].float()).view(tokens, heads, vdim)
@@ -366,8 +405,12 @@ class TorchKernels:
             weights = weights / (weights.sum(-1, keepdim=True) + 1e-20)
         return chosen.to(torch.int32), (weights * scale).float()
 
-    def prepare_experts(self, ups, downs, activation, gates=None):
+    def prepare_experts(self, ups, downs, activation, gates=None, limit=None):
         stacked = torch.stack([w.float() for w in gates]) if gates is not None else None
+        if activation == "limited_swish":
+            if stacked is None or limit is None or not limit > 0:
+                raise ValueError("experts: limited_swish gates an expert and has a positive limit")
+            activation = ("limited_swish", float(limit))
         return (torch.stack([w.float() for w in ups]), torch.stack([w.float() for w in downs]), activation, stacked)
 
     def conv_gated_delta_rule(self, projected, channels, taps, activation, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, window, state,
@@ -383,6 +426,10 @@ class TorchKernels:
                 e = int(chosen[t, slot])
                 if gate_weights is None:
                     inner = self.activate((x[t].float() @ ups[e].T).to(self.dtype), activation).float()
+                elif isinstance(activation, tuple):  # a function of gate and up both, rounded to the run dtype before
+                    gate = (x[t].float() @ gate_weights[e].T).to(self.dtype).float()
+                    up = (x[t].float() @ ups[e].T).to(self.dtype).float()
+                    inner = _limited_swish(gate, up, activation[1]).to(self.dtype).float()
                 else:  # act(gate x) * (up x), both rounded to the run dtype before
                     gate = self.activate((x[t].float() @ gate_weights[e].T).to(self.dtype), activation).float()
                     inner = (gate * (x[t].float() @ ups[e].T).to(self.dtype).float()).to(self.dtype).float()
