@@ -143,13 +143,26 @@ def retention_mixer(h, positions, m, t, prefix, eps):
     k = k * dim ** -0.5
     read = torch.zeros((n, heads, vdim), dtype=F)
     for head in range(heads):
-        state = torch.zeros((dim, vdim), dtype=F)
-        decay = float(m["decay"][head])
-        for step in range(n):
-            state = decay * state + torch.outer(k[step, head], v[step, head])
-            read[step, head] = state.T @ q[step, head]
+        read[:, head] = retention_head(q[:, head], k[:, head], v[:, head], float(m["decay"][head]))
     read = rms_normalise(read, eps).reshape(n, heads * vdim)
     return (read * silu(h @ t[prefix + "g"].T)) @ t[prefix + "o"].T
+
+
+def retention_head(q, k, v, decay):
+    """S_t = decay S_(t-1) + k_t v_t^T from S = 0, o_t = S_t^T q_t, for one head: q, k [n, d], v [n, dv].  Short
+    sequences token by token, as the recurrence is written; long ones by its closed form, o_t = sum over s <= t of
+    decay^(t-s) (q_t . k_s) v_s, which is the same sum."""
+    n = q.shape[0]
+    if n <= 48:
+        state = torch.zeros((q.shape[1], v.shape[1]), dtype=F)
+        out = torch.zeros((n, v.shape[1]), dtype=F)
+        for step in range(n):
+            state = decay * state + torch.outer(k[step], v[step])
+            out[step] = state.T @ q[step]
+        return out
+    distance = (torch.arange(n)[:, None] - torch.arange(n)[None, :]).clamp(min=0).to(F)
+    fade = torch.tril(torch.tensor(decay, dtype=F) ** distance)
+    return ((q @ k.T) * fade) @ v
 
 
 def latent_mixer(h, positions, m, t, prefix, eps):
@@ -192,11 +205,11 @@ def expert_feed_forward(h, mlp, t, prefix):
     best, chosen = torch.topk(logits, router["top"], dim=-1)
     weights = torch.softmax(best, dim=-1)
     out = torch.zeros_like(h)
-    for row in range(h.shape[0]):
-        for weight, expert in zip(weights[row], chosen[row].tolist()):
-            name = f"{prefix}e{expert}."
-            y = limited_gate(h[row] @ t[name + "gate"].T, h[row] @ t[name + "up"].T, limit)
-            out[row] += weight * (y @ t[name + "down"].T)
+    for expert in range(router["experts"]):
+        name = f"{prefix}e{expert}."
+        share = (weights * (chosen == expert)).sum(-1, keepdim=True)  # the token's weight for this expert, 0 if it is not chosen
+        y = limited_gate(h @ t[name + "gate"].T, h @ t[name + "up"].T, limit)
+        out += share * (y @ t[name + "down"].T)
     return out
 
 
