@@ -38,6 +38,11 @@ does the same for the third (configs/sozavik-w1536.json, configs/sozavik-w3584.j
 
 measures the fourth (configs/katenex-w1536.json, configs/katenex-w3584.json) beside the Dafutar models of the same width
 and number of layer runs (the engine's other decoder with the delta rule and routed experts) and the Qwen2 models.
+
+    python bench.py --op vagozen
+
+measures the fifth (configs/vagozen-w1536.json, configs/vagozen-w3584.json) beside the Sozavik models (window attention, a
+decaying state, norms behind the sublayers), the Dafutar models (latent attention, experts, layers walked twice) and the Qwen2 models.
 """
 
 from __future__ import annotations
@@ -79,7 +84,7 @@ def parse() -> argparse.Namespace:
                         help="leave out decoding at contexts of 8k and 30k (batch 8) and 4k (batch 64), and the long prompts")
     parser.add_argument("--skip-other-models", action="store_true",
                         help="leave out the float32 run and the 7B and 32B layer sizes")
-    parser.add_argument("--op", choices=("decode-attention", "prefill-attention", "dafutar", "sozavik", "katenex"), default=None,
+    parser.add_argument("--op", choices=("decode-attention", "prefill-attention", "dafutar", "sozavik", "katenex", "vagozen"), default=None,
                         help="measure one operation alone instead, as the reference's kernel benchmark does")
     return parser.parse_args()
 
@@ -434,6 +439,8 @@ def main() -> int:
         return sozavik_table(args)
     if args.op == "katenex":
         return katenex_table(args)
+    if args.op == "vagozen":
+        return vagozen_table(args)
 
     import torch
 
@@ -582,6 +589,14 @@ def katenex_table(args) -> int:
     softmax attention beside a gated linear recurrence; experts chosen within groups) at two layer sizes beside the
     Dafutar and the Qwen2 of the same width, number of layer runs and vocabulary, measured as `dafutar_table` measures."""
     return beside_qwen2(args, "katenex", "Katenex", also=("dafutar",))
+
+
+def vagozen_table(args) -> int:
+    """The Vagozen decoder (a norm before and behind every sublayer; layers of window attention that keeps a sequence's
+    first tokens, of retention and of latent attention; a gate with a limit, dense and in experts; layers walked twice) at
+    two layer sizes beside the Sozavik, the Dafutar and the Qwen2 of the same width, number of layer runs and vocabulary,
+    measured as `dafutar_table` measures."""
+    return beside_qwen2(args, "vagozen", "Vagozen", also=("sozavik", "dafutar"))
 
 
 def beside_qwen2(args, name: str, title: str, also: tuple[str, ...] = ()) -> int:

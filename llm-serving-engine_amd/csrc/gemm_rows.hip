@@ -18,6 +18,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define ACT_GELU 1
 #define ACT_GELU_TANH 2
 #define ACT_RELU 3
+// a function of gate and up both, with a limit (gated results only): g = min(gate, limit), u = clamp(up, -limit, limit),
+// g * sigmoid(1.702 g) * (u + 1)
+#define ACT_LIMITED_SWISH 4
 
 __device__ __forceinline__ float activation_of(int activation, float z) {
   switch (activation) {
@@ -36,7 +39,8 @@ __device__ __forceinline__ float activation_of(int activation, float z) {
 
 // A lane's four neighbouring columns n0 .. n0 + 3 (n0 a multiple of four) of a row of a product `outputs` wide.
 template <typename TO>
-__device__ __forceinline__ void store_four(TO* __restrict__ out, size_t row, int n0, int outputs, int activation, const f32x4& v) {
+__device__ __forceinline__ void store_four(TO* __restrict__ out, size_t row, int n0, int outputs, int activation, const f32x4& v,
+                                           float limit = 0.f) {
   if (activation < ACT_GATED) {
     TO* dst = out + row * outputs;
 #pragma unroll
@@ -50,7 +54,12 @@ __device__ __forceinline__ void store_four(TO* __restrict__ out, size_t row, int
     const int n = n0 + 2 * pair;
     if (n + 1 < outputs) {
       const float gate = to_float(from_float<TO>(v[2 * pair])), up = to_float(from_float<TO>(v[2 * pair + 1]));
-      dst[n / 2] = from_float<TO>(activation_of(activation - ACT_GATED, gate) * up);
+      if (activation - ACT_GATED == ACT_LIMITED_SWISH) {
+        const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+        dst[n / 2] = from_float<TO>(g / (1.f + expf(-1.702f * g)) * (u + 1.f));
+      } else {
+        dst[n / 2] = from_float<TO>(activation_of(activation - ACT_GATED, gate) * up);
+      }
     }
   }
 }
@@ -150,7 +159,7 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16_t* __rest
 template <int NT, int MT, typename TO>
 __global__ __launch_bounds__(256) void expert_product_mfma_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order, int top,
                                                                   const bf16_t* __restrict__ w, int outputs, int inner,
-                                                                  const int* __restrict__ tiles, TO* __restrict__ out, int activation) {
+                                                                  const int* __restrict__ tiles, TO* __restrict__ out, int activation, float limit) {
   const int* tile = tiles + 3 * (size_t)blockIdx.y;
   const int expert = tile[0], first = tile[1], rows = tile[2];
   if (rows == 0) return;
@@ -184,7 +193,7 @@ __global__ __launch_bounds__(256) void expert_product_mfma_kernel(const bf16_t* 
     const int m = t * 16 + r;
     if (m >= rows) continue;
 #pragma unroll
-    for (int s = 0; s < NT; ++s) store_four<TO>(out, (size_t)(first + m), col0 + s * 16 + g * 4, outputs, activation, acc[s][t]);
+    for (int s = 0; s < NT; ++s) store_four<TO>(out, (size_t)(first + m), col0 + s * 16 + g * 4, outputs, activation, acc[s][t], limit);
   }
 }
 
@@ -199,7 +208,7 @@ __global__ __launch_bounds__(256) void expert_product_mfma_kernel(const bf16_t* 
 template <typename TO>
 __global__ __launch_bounds__(256) void expert_tiled_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order, int top,
                                                            const bf16_t* __restrict__ w, int outputs, int inner,
-                                                           const int* __restrict__ tiles, TO* __restrict__ out, int activation) {
+                                                           const int* __restrict__ tiles, TO* __restrict__ out, int activation, float limit) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[TILED_ROWS * TILED_LINE], ws[TILED_ROWS * TILED_LINE];
   const int* tile = tiles + 3 * (size_t)blockIdx.y;
   const int expert = tile[0], first = tile[1], rows = tile[2];
@@ -265,7 +274,7 @@ __global__ __launch_bounds__(256) void expert_tiled_kernel(const bf16_t* __restr
     const int m = wave_row + u * 16 + r;
     if (m >= rows) continue;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) store_four<TO>(out, (size_t)(first + m), col0 + wave_col + s * 16 + g * 4, outputs, activation, acc[s][u]);
+    for (int s = 0; s < 4; ++s) store_four<TO>(out, (size_t)(first + m), col0 + wave_col + s * 16 + g * 4, outputs, activation, acc[s][u], limit);
   }
 }
 
@@ -276,7 +285,7 @@ __global__ __launch_bounds__(256) void expert_tiled_kernel(const bf16_t* __restr
 template <typename TO>
 __global__ __launch_bounds__(256) void expert_stream_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order, int top,
                                                             const bf16_t* __restrict__ w, int outputs, int inner,
-                                                            const int* __restrict__ tiles, TO* __restrict__ out, int activation) {
+                                                            const int* __restrict__ tiles, TO* __restrict__ out, int activation, float limit) {
   __shared__ f32x4 partial[4][WAVE];
   const int* tile = tiles + 3 * (size_t)blockIdx.y;
   const int expert = tile[0], first = tile[1], rows = tile[2];
@@ -304,7 +313,7 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(const bf16_t* __rest
   f32x4 total = partial[0][lane];
 #pragma unroll
   for (int v = 1; v < 4; ++v) total += partial[v][lane];
-  store_four<TO>(out, (size_t)(first + r), blockIdx.x * 16 + g * 4, outputs, activation, total);
+  store_four<TO>(out, (size_t)(first + r), blockIdx.x * 16 + g * 4, outputs, activation, total, limit);
 }
 
 // ---------------------------------------------------------------------------- a product per head
@@ -571,8 +580,9 @@ extern "C" int llmserve_expert_product_gates(int is_float, int inner, int tile_r
 
 extern "C" int llmserve_expert_product(const void* x, int is_float, const int* order, int top, const void* w, int outputs,
                                        int inner, const int* tiles, int capacity, int tile_rows, void* out, int out_is_float,
-                                       int activation, hipStream_t stream) {
+                                       int activation, float limit, hipStream_t stream) {
   if (capacity <= 0) return 0;
+  if ((activation == ACT_GATED + ACT_LIMITED_SWISH && !(limit > 0.f)) || activation == ACT_LIMITED_SWISH) return ERR_BAD_ARGUMENT;
   if (capacity > 65535 || outputs < 1 || inner < 1) return ERR_BAD_ARGUMENT;
   // a gated result comes from the matrix-core kernels alone, of an even number of columns
   if (activation >= ACT_GATED && (outputs % 2 || !llmserve_expert_product_gates(is_float, inner, tile_rows))) return ERR_BAD_ARGUMENT;
@@ -581,10 +591,10 @@ extern "C" int llmserve_expert_product(const void* x, int is_float, const int* o
     const dim3 through_lds((outputs + TILED_ROWS - 1) / TILED_ROWS, capacity);
     if (out_is_float)
       hipLaunchKernelGGL(expert_tiled_kernel<float>, through_lds, dim3(256), 0, stream, (const bf16_t*)x, order, top, (const bf16_t*)w,
-                         outputs, inner, tiles, (float*)out, activation);
+                         outputs, inner, tiles, (float*)out, activation, limit);
     else
       hipLaunchKernelGGL(expert_tiled_kernel<bf16_t>, through_lds, dim3(256), 0, stream, (const bf16_t*)x, order, top, (const bf16_t*)w,
-                         outputs, inner, tiles, (bf16_t*)out, activation);
+                         outputs, inner, tiles, (bf16_t*)out, activation, limit);
     return LAUNCH_STATUS();
   }
   if (!is_float && inner % 32 == 0) {
@@ -593,10 +603,10 @@ extern "C" int llmserve_expert_product(const void* x, int is_float, const int* o
       const dim3 streams((outputs + 15) / 16, capacity);
       if (out_is_float)
         hipLaunchKernelGGL(expert_stream_kernel<float>, streams, dim3(256), 0, stream, (const bf16_t*)x, order, top, (const bf16_t*)w,
-                           outputs, inner, tiles, (float*)out, activation);
+                           outputs, inner, tiles, (float*)out, activation, limit);
       else
         hipLaunchKernelGGL(expert_stream_kernel<bf16_t>, streams, dim3(256), 0, stream, (const bf16_t*)x, order, top, (const bf16_t*)w,
-                           outputs, inner, tiles, (bf16_t*)out, activation);
+                           outputs, inner, tiles, (bf16_t*)out, activation, limit);
       return LAUNCH_STATUS();
     }
     const int nt = outputs <= 64 ? 1 : outputs <= 128 ? 2 : 4;
@@ -605,10 +615,10 @@ extern "C" int llmserve_expert_product(const void* x, int is_float, const int* o
   do {                                                                                                                          \
     if (out_is_float)                                                                                                           \
       hipLaunchKernelGGL((expert_product_mfma_kernel<NT, MT, float>), cores, dim3(256), 0, stream, (const bf16_t*)x, order, top, \
-                         (const bf16_t*)w, outputs, inner, tiles, (float*)out, activation);                                     \
+                         (const bf16_t*)w, outputs, inner, tiles, (float*)out, activation, limit);                              \
     else                                                                                                                        \
       hipLaunchKernelGGL((expert_product_mfma_kernel<NT, MT, bf16_t>), cores, dim3(256), 0, stream, (const bf16_t*)x, order, top, \
-                         (const bf16_t*)w, outputs, inner, tiles, (bf16_t*)out, activation);                                    \
+                         (const bf16_t*)w, outputs, inner, tiles, (bf16_t*)out, activation, limit);                             \
   } while (0)
     if (tile_rows == 64) {
       if (nt == 1) LAUNCH_EXPERTS(1, 4); else if (nt == 2) LAUNCH_EXPERTS(2, 4); else LAUNCH_EXPERTS(4, 4);

@@ -231,17 +231,19 @@ extern "C" int llmserve_add_normed_norm(float* hidden, const float* update, int 
 // ---------------------------------------------------------------------------- heads turned in place
 // For every token and every one of `heads` heads (`head_stride` columns each, from column `first` of a row `x_width`
 // wide): the first `dims` columns turn in pairs (pairing 1: (2i, 2i + 1); 2: (i, i + dims / 2)) by (cos, sin) of
-// table[token][i], and every column of the head is multiplied by `scale`.  float32 arithmetic; a thread a pair, or a
-// column beyond the pairs.
+// table[token][i], and every column of a head from head `scale_from` on is multiplied by `scale` (queries and keys side by
+// side are one launch, the keys scaled).  float32 arithmetic; a thread a pair, or a column beyond the pairs.
 template <typename T>
 __global__ __launch_bounds__(256) void rotate_heads_kernel(T* __restrict__ x, int x_width, int first, int head_stride, int heads,
-                                                           const float* __restrict__ table, int dims, int pairing, float scale) {
+                                                           const float* __restrict__ table, int dims, int pairing, float scale_of_some,
+                                                           int scale_from) {
   const size_t token = blockIdx.x;
   T* row = x + token * x_width + first;
   const int half = dims / 2, per_head = head_stride - half;  // work items a head: the pairs, then the columns left
   for (int item = threadIdx.x; item < heads * per_head; item += blockDim.x) {
     const int head = item / per_head, inside = item - head * per_head;
     T* at = row + (size_t)head * head_stride;
+    const float scale = head >= scale_from ? scale_of_some : 1.f;
     if (inside < half) {
       const int a_at = pairing == 1 ? 2 * inside : inside, b_at = pairing == 1 ? 2 * inside + 1 : inside + half;
       const float2 cs = ((const float2*)table)[token * half + inside];
@@ -256,17 +258,17 @@ __global__ __launch_bounds__(256) void rotate_heads_kernel(T* __restrict__ x, in
 }
 
 extern "C" int llmserve_rotate_heads(void* x, int is_float, int tokens, int x_width, int first, int head_stride, int heads,
-                                     const float* table, int dims, int pairing, float scale, hipStream_t stream) {
+                                     const float* table, int dims, int pairing, float scale, int scale_from, hipStream_t stream) {
   if (tokens <= 0 || heads <= 0) return 0;
   if (dims < 0 || dims % 2 || dims > head_stride || first < 0 || first + heads * head_stride > x_width || (dims > 0 && !table) ||
       (dims > 0 && pairing != 1 && pairing != 2))
     return ERR_BAD_ARGUMENT;
   if (is_float)
     hipLaunchKernelGGL(rotate_heads_kernel<float>, dim3(tokens), dim3(256), 0, stream, (float*)x, x_width, first, head_stride, heads,
-                       table, dims, pairing, scale);
+                       table, dims, pairing, scale, scale_from);
   else
     hipLaunchKernelGGL(rotate_heads_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (bf16_t*)x, x_width, first, head_stride, heads,
-                       table, dims, pairing, scale);
+                       table, dims, pairing, scale, scale_from);
   return LAUNCH_STATUS();
 }
 

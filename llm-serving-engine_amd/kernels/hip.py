@@ -56,7 +56,7 @@ _SIGNATURES = {
     "llmserve_gate_mul": "pipiiiip",
     "llmserve_gate_mul_limit": "pipiiiifp",
     "llmserve_add_normed_norm": "ppipifpifpiiip",
-    "llmserve_rotate_heads": "piiiiiipiifp",
+    "llmserve_rotate_heads": "piiiiiipiifip",
     "llmserve_add_rows": "ppippiip",
     "llmserve_gather_rows": "ppiippiip",
     "llmserve_gemm_generic": "pipipipiiiip",
@@ -87,7 +87,7 @@ _SIGNATURES = {
     "llmserve_headwise_linear": "piiiiipiiipiiip",
     "llmserve_route": "piipifppiiiiip",
     "llmserve_sort_pairs": "piipppiip",
-    "llmserve_expert_product": "pipipiipiipiip",
+    "llmserve_expert_product": "pipipiipiipiifp",
     "llmserve_expert_product_gates": "iii",
     "llmserve_combine_pairs": "pppipiippiip",
     "llmserve_conv_gated_delta_rule": "piiipipppppiiiippiiippppppip",
@@ -1252,13 +1252,12 @@ class HipKernels:
         _check(library.llmserve_sort_pairs(_pointer(chosen), pairs, count, _pointer(place), _pointer(order), _pointer(tiles), capacity, tile_rows, self._stream), "experts: sort")
         # the matrix-core kernels gate their result themselves (act(gate) * up of neighbouring columns); behind the others a
         # kernel of its own does
-        # (the gate with a limit is a function of gate and up both: the kernel behind the product applies it)
-        fused = gated and activation != "limited_swish" and bool(library.llmserve_expert_product_gates(_is_float(x), hidden, tile_rows))
+        fused = gated and bool(library.llmserve_expert_product_gates(_is_float(x), hidden, tile_rows))
         code = _ACTIVATIONS[activation] + _GATED_RESULT if fused else -1 if gated else _ACTIVATIONS[activation]
         inner = self._empty((pairs, width if fused else size), x.dtype)
         _check(library.llmserve_expert_product(
             _pointer(x), _is_float(x), _pointer(order), top, _pointer(ups), size, hidden, _pointer(tiles), capacity, tile_rows, _pointer(inner),
-            _is_float(inner), code, self._stream), "experts: first product")
+            _is_float(inner), code, limit, self._stream), "experts: first product")
         if gated and not fused:
             both = inner
             inner = self._empty((pairs, width), x.dtype)
@@ -1268,7 +1267,7 @@ class HipKernels:
         rows = self._empty((pairs, hidden), torch.float32)
         _check(library.llmserve_expert_product(
             _pointer(inner), _is_float(inner), _pointer(order), 0, _pointer(downs), hidden, size, _pointer(tiles), capacity, tile_rows, _pointer(rows),
-            1, -1, self._stream), "experts: second product")
+            1, -1, 0.0, self._stream), "experts: second product")
         if shared is not None and (shared.dtype != torch.float32 or shared.shape != (tokens, hidden) or (gates is not None and gates.dtype != torch.float32)):
             raise KernelError("experts: the shared rows and their gates are float32")
         out = self._empty((tokens, hidden), torch.float32)
@@ -1416,13 +1415,13 @@ class HipKernels:
         _check(status, "add_normed_norm")
         return out
 
-    def rotate_heads(self, x, first: int, head_stride: int, heads: int, table, dims: int, pairing: str, scale: float = 1.0) -> torch.Tensor:
+    def rotate_heads(self, x, first: int, head_stride: int, heads: int, table, dims: int, pairing: str, scale: float = 1.0, scale_from: int = 0) -> torch.Tensor:
         tokens = x.shape[0]
         if dims and (pairing not in ("adjacent", "half") or table is None or table.dtype != torch.float32 or table.shape != (tokens, dims // 2, 2)):
             raise KernelError("rotate_heads: pairs that are adjacent or halves apart, and a float32 table entry for every pair of every token")
         status = self._library_of("heads").llmserve_rotate_heads(
             _pointer(x), _is_float(x), tokens, x.shape[1], first, head_stride, heads, _pointer(table if dims else None), dims,
-            _PAIRINGS[pairing] if dims else 0, float(scale), self._stream,
+            _PAIRINGS[pairing] if dims else 0, float(scale), int(scale_from), self._stream,
         )
         _check(status, "rotate_heads")
         return x

@@ -176,11 +176,12 @@ class Kernels(Protocol):
 
     def rotate_heads(
         self, x: torch.Tensor, first: int, head_stride: int, heads: int, table: torch.Tensor | None, dims: int, pairing: str, scale: float = 1.0,
+        scale_from: int = 0,
     ) -> torch.Tensor:
         """In place, for `heads` heads of `head_stride` columns from column `first` of x's rows (float32 or the run
         dtype): the first `dims` columns of a head turn in pairs (`pairing` "adjacent": (2i, 2i + 1); "half": (i, i +
-        dims / 2)) by the token's row of `table` (float32 [T, dims / 2, 2], cos and sin), and the whole head is multiplied
-        by `scale`; float32 arithmetic."""
+        dims / 2)) by the token's row of `table` (float32 [T, dims / 2, 2], cos and sin), and every head from head `scale_from`
+        on is multiplied by `scale` (queries and keys side by side in one call, the keys scaled); float32 arithmetic."""
 
     def add_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None, other: torch.Tensor | None, vector: torch.Tensor | None) -> torch.Tensor:
         """`hidden += delta (its parts added in order) + other + vector` in place, float32: `other` rows of the stream's

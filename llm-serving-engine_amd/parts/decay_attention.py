@@ -97,8 +97,8 @@ class DecayAttention(Mixer):
         projected = kernels.linear(x, self.inputs, out_dtype=torch.float32 if self.turned else None)  # [T, q | k | v | g]
         if self.turned:
             table = kernels.rotary_table(batch, self.frequencies) if spec.rot_dims else None
-            kernels.rotate_heads(projected, 0, spec.dim, heads, table, spec.rot_dims, spec.pairing, 1.0)
-            kernels.rotate_heads(projected, qk, spec.dim, heads, table, spec.rot_dims, spec.pairing, spec.key_scale)
+            # (queries and keys lie side by side: one call, the keys scaled)
+            kernels.rotate_heads(projected, 0, spec.dim, 2 * heads, table, spec.rot_dims, spec.pairing, spec.key_scale, scale_from=heads)
         read = kernels.decay_attention(
             projected, 0, qk, 2 * qk, heads, spec.dim, spec.vdim, self.decays, spec.activation, batch, cell.state
         )  # float32 [T, heads * vdim]

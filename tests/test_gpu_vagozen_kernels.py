@@ -56,9 +56,10 @@ def test_rotate_heads(kernels, dtype, pairing, heads, stride, dims, scale):
     table = torch.stack([angles.cos(), angles.sin()], dim=-1)[:, : dims // 2].contiguous()
     for kind in (torch.float32, dtype):  # (rows a product left in float32, and rows in the run dtype)
         x = torch.randn(tokens, first + heads * stride + 3).to(kind)
-        want = TorchKernels(dtype).rotate_heads(x.clone(), first, stride, heads, table, dims, pairing, scale)
-        got = kernels[dtype].rotate_heads(gpu(x), first, stride, heads, gpu(table) if dims else None, dims, pairing, scale)
-        close(got, want, kind)
+        for scale_from in (0, heads // 2):
+            want = TorchKernels(dtype).rotate_heads(x.clone(), first, stride, heads, table, dims, pairing, scale, scale_from)
+            got = kernels[dtype].rotate_heads(gpu(x), first, stride, heads, gpu(table) if dims else None, dims, pairing, scale, scale_from)
+            close(got, want, kind)
         assert torch.equal(got.cpu()[:, :first], x[:, :first]) and torch.equal(got.cpu()[:, first + heads * stride:], x[:, first + heads * stride:])
 
 

@@ -340,7 +340,7 @@ class TorchKernels:
         x.copy_((x.float().view(x.shape[0], heads, width) * gate[:, :, None]).reshape(x.shape).to(x.dtype))
         return x
 
-    def rotate_heads(self, x, first, head_stride, heads, table, dims, pairing, scale=1.0):
+    def rotate_heads(self, x, first, head_stride, heads, table, dims, pairing, scale=1.0, scale_from=0):
         tokens = x.shape[0]
         for head in range(heads):
             part = x[:, first + head * head_stride : first + (head + 1) * head_stride].float()
@@ -350,7 +350,7 @@ class TorchKernels:
                 a, b = part[:, one].clone(), part[:, two].clone()
                 part[:, one] = a * cos - b * sin
                 part[:, two] = b * cos + a * sin
-            x[:, first + head * head_stride : first + (head + 1) * head_stride] = (part * scale).to(x.dtype)
+            x[:, first + head * head_stride : first + (head + 1) * head_stride] = (part * (scale if head >= scale_from else 1.0)).to(x.dtype)
         return x
 
     def add_normed_norm(self, hidden, update, weight, eps, next_weight, next_eps):
@@ -421,19 +421,24 @@ class TorchKernels:
     def expert_feed_forward(self, x, experts, chosen, weights, shared=None, gates=None, gate_column=0):
         ups, downs, activation, gate_weights = experts
         out = torch.zeros((x.shape[0], downs.shape[1]))
-        for t in range(x.shape[0]):
-            for slot in range(chosen.shape[1]):
-                e = int(chosen[t, slot])
-                if gate_weights is None:
-                    inner = self.activate((x[t].float() @ ups[e].T).to(self.dtype), activation).float()
-                elif isinstance(activation, tuple):  # a function of gate and up both, rounded to the run dtype before
-                    gate = (x[t].float() @ gate_weights[e].T).to(self.dtype).float()
-                    up = (x[t].float() @ ups[e].T).to(self.dtype).float()
-                    inner = _limited_swish(gate, up, activation[1]).to(self.dtype).float()
-                else:  # act(gate x) * (up x), both rounded to the run dtype before
-                    gate = self.activate((x[t].float() @ gate_weights[e].T).to(self.dtype), activation).float()
-                    inner = (gate * (x[t].float() @ ups[e].T).to(self.dtype).float()).to(self.dtype).float()
-                out[t] += weights[t, slot] * (inner @ downs[e].T)
+        rows = torch.zeros((x.shape[0], chosen.shape[1], downs.shape[1]))  # every (token, choice) pair's row, then added in the order of the choices
+        for e in range(ups.shape[0]):
+            tokens, slots = (chosen == e).nonzero(as_tuple=True)
+            if tokens.numel() == 0:
+                continue
+            mine = x[tokens].float()
+            if gate_weights is None:
+                inner = self.activate((mine @ ups[e].T).to(self.dtype), activation).float()
+            elif isinstance(activation, tuple):  # a function of gate and up both, rounded to the run dtype before
+                gate = (mine @ gate_weights[e].T).to(self.dtype).float()
+                up = (mine @ ups[e].T).to(self.dtype).float()
+                inner = _limited_swish(gate, up, activation[1]).to(self.dtype).float()
+            else:  # act(gate x) * (up x), both rounded to the run dtype before
+                gate = self.activate((mine @ gate_weights[e].T).to(self.dtype), activation).float()
+                inner = (gate * (mine @ ups[e].T).to(self.dtype).float()).to(self.dtype).float()
+            rows[tokens, slots] = inner @ downs[e].T
+        for slot in range(chosen.shape[1]):
+            out += weights[:, slot : slot + 1] * rows[:, slot]
         if shared is not None:
             out += torch.sigmoid(gates[:, gate_column : gate_column + 1].float()) * shared if gates is not None else shared
         return out
