@@ -893,11 +893,12 @@ class HipKernels:
         store inside the same kernel.  With `unmerged` (a step of single tokens whose reader merges
         key splits itself) the keys are split more finely and the splits are returned as they are
         (their results in bfloat16, laid out for `gemm_merged`; their maxima and sums in float32; how
-        many), instead of `out`.  `changed` = (slopes or None, soft cap or 0.0, sinks or None): scores changed before
-        the softmax or a sink in its denominator, which neither `fuse` nor the kernel that shares keys through LDS takes."""
+        many), instead of `out`.  `changed` = (slopes or None, soft cap or 0.0, sinks or None, kept first keys or 0): scores
+        changed before the softmax, a sink in its denominator, or a sequence's first keys kept visible behind the window, which neither
+        `fuse` nor the kernel that shares keys through LDS takes."""
         if changed is not None and fuse is not None:
             raise KernelError("paged_attention: the fused decode form takes plain scores only")
-        slopes, soft_cap, sinks, keep_first = (*changed, 0)[:4] if changed is not None else (None, 0.0, None, 0)
+        slopes, soft_cap, sinks, keep_first = changed if changed is not None else (None, 0.0, None, 0)
         library = self._attention_library(layout.head_dim)
         heads, kv_heads = layout.num_heads, layout.num_kv_heads
         per_tile = max(1, 16 // (heads // kv_heads))
