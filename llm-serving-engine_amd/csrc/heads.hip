@@ -235,7 +235,7 @@ extern "C" int llmserve_add_normed_norm(float* hidden, const float* update, int 
 // side are one launch, the keys scaled).  float32 arithmetic; a thread a pair, or a column beyond the pairs.
 template <typename T>
 __global__ __launch_bounds__(256) void rotate_heads_kernel(T* __restrict__ x, int x_width, int first, int head_stride, int heads,
-                                                           const float* __restrict__ table, int dims, int pairing, float scale_of_some,
+                                                           const float* __restrict__ table, int dims, int pairing, float later_scale,
                                                            int scale_from) {
   const size_t token = blockIdx.x;
   T* row = x + token * x_width + first;
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256) void rotate_heads_kernel(T* __restrict__ x, in
   for (int item = threadIdx.x; item < heads * per_head; item += blockDim.x) {
     const int head = item / per_head, inside = item - head * per_head;
     T* at = row + (size_t)head * head_stride;
-    const float scale = head >= scale_from ? scale_of_some : 1.f;
+    const float scale = head >= scale_from ? later_scale : 1.f;
     if (inside < half) {
       const int a_at = pairing == 1 ? 2 * inside : inside, b_at = pairing == 1 ? 2 * inside + 1 : inside + half;
       const float2 cs = ((const float2*)table)[token * half + inside];
